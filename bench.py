@@ -1,0 +1,261 @@
+#!/usr/bin/env python3
+"""Benchmark of the Winograd-ReLU conv layer (winograd2x2_imTrans + winograd2x2_conv) on one MI355X.
+
+A step is one pass of the hot path over one synthetic batch, inputs resident in HBM:
+  TI = winograd2x2_imTrans(x, relu)      [B,H,W,C] -> [16,B,nH,nW,C]
+  y  = winograd2x2_conv(TI, W)           [16,B,nH,nW,C] x [16,C,K] -> [B,2nH,2nW,K]
+Default workload: ResNet-18 conv3 stage, N=64, 28x28x128 -> 128, fp32, Winograd-domain ReLU
+on, weights magnitude-pruned to 20 % density (values only: the contraction is dense, as in
+the reference, winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_cuda.cu.cc:80-85).
+
+Prints one JSON line.  `value` is the effective direct-convolution rate 18*N*H*W*C*K / step
+time.  `roofline` describes the MFMA kernel (32*M*C*K flop per launch), `roofline_imtrans`
+the transform kernel (4*B*H*W*C + 64*M*C bytes per launch); both use the average launch
+duration measured with HIP events on the launching stream.  `cpu_baseline` times the CPU
+oracle (OpenMP C restatement of the same three stages) on this host's cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "sparse-winograd-cnn_amd")
+for _p in (ROOT, PKG):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, datasheet
+FP32_MFMA_PEAK_TF = 157.3  # MI355X dense fp32 matrix, datasheet
+BF16_MFMA_PEAK_TF = 2500.0
+
+# name: (B, H, W, C, K, weight density, input kind)
+WORKLOADS = {
+    "cfg1": (1, 16, 16, 64, 64, 1.0, "normal"),
+    "cfg2": (64, 56, 56, 64, 64, 0.3, "halfnormal"),
+    "cfg3": (64, 28, 28, 128, 128, 0.2, "normal"),
+    "cfg4a": (64, 14, 14, 256, 256, 0.1, "normal"),
+    "cfg4b": (64, 7, 7, 512, 512, 0.1, "normal"),
+}
+SEEDS = {"cfg1": 100, "cfg2": 200, "cfg3": 300, "cfg4a": 400, "cfg4b": 410}
+
+
+def make_inputs(name):
+    import numpy as np
+    from winograd_weights import gen_prune_mask
+
+    B, H, W, C, K, density, kind = WORKLOADS[name]
+    seed = SEEDS[name]
+    x = np.random.default_rng(seed).standard_normal((B, H, W, C)).astype(np.float32)
+    if kind == "halfnormal":
+        x = np.maximum(x, 0)
+    w = (np.random.default_rng(seed + 1).standard_normal((16, C, K)) * 0.05).astype(np.float32)
+    if density < 1.0:
+        gen_prune_mask(w, density)
+    return x, w
+
+
+def time_loop(fn, iters, torch):
+    """Average duration of `iters` back-to-back calls, by HIP events on the current stream (ms)."""
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def cpu_baseline(name, x, w, budget_s):
+    """The oracle's three stages on the host cores; returns (dict, ti_ref, y_ref)."""
+    import numpy as np
+
+    import oracle
+
+    B, H, W, C, K = WORKLOADS[name][:5]
+    nH, nW = (H + 1) // 2, (W + 1) // 2
+    flops = 18.0 * B * H * W * C * K
+    times, stages = [], None
+    t_begin = time.perf_counter()
+    ti = y = None
+    while True:
+        t0 = time.perf_counter()
+        ti = oracle.imtrans(x, relu=True)
+        t1 = time.perf_counter()
+        p = oracle.gemm16(ti, w)
+        t2 = time.perf_counter()
+        y = oracle.output_transform(p, B, nH, nW)
+        t3 = time.perf_counter()
+        times.append(t3 - t0)
+        if stages is None or t3 - t0 <= min(times):
+            stages = (t1 - t0, t2 - t1, t3 - t2)
+        if len(times) >= 9 or (time.perf_counter() - t_begin) > budget_s and len(times) >= 3:
+            break
+    med = float(np.median(times))
+    return {
+        "value": round(flops / med / 1e9, 2),
+        "unit": "GFLOP/s",
+        "cores": oracle.num_threads(),
+        "kind": "port",
+        "sample": "%d full %s steps (whole batch), median; best-step stages imtrans/gemm/output = %.1f/%.1f/%.1f ms"
+                  % (len(times), name, stages[0] * 1e3, stages[1] * 1e3, stages[2] * 1e3),
+        "ms_per_step": round(med * 1e3, 2),
+    }, ti, y
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg and the parity gate")
+    ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU work for cpu_baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this path runs on one GPU only; --gpus %d is not supported (the forward pass "
+                 "shards over the batch with no exchange step, so N GPUs are N independent copies of this run)"
+                 % args.gpus)
+
+    import numpy as np
+    import torch
+
+    import swc_hip
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv
+    from winograd2x2_imTrans.winograd2x2_imTrans import winograd2x2_imTrans
+
+    swc_hip.lib()  # fail loudly if the HIP library is not built
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    prop = torch.cuda.get_device_properties(dev)
+    print("device: %s, %d CUs, %.0f MHz, %.0f GiB" % (prop.name, prop.multi_processor_count,
+          getattr(prop, "clock_rate", 0) / 1e3, prop.total_memory / 2 ** 30), file=sys.stderr)
+
+    name = args.workload
+    B, H, W, C, K, density, kind = WORKLOADS[name]
+    nH, nW = (H + 1) // 2, (W + 1) // 2
+    M = B * nH * nW
+    x_np, w_np = make_inputs(name)
+    x = torch.from_numpy(x_np).to(dev)
+    w = torch.from_numpy(w_np).to(dev)
+    ti = torch.empty(16, B, nH, nW, C, device=dev)
+    y = torch.empty(B, 2 * nH, 2 * nW, K, device=dev)
+
+    # The timed loop calls the launcher-level C entry points directly with prebuilt arguments
+    # (the Python op wrappers re-validate shapes on every call, which costs more host time
+    # than the transform kernel runs for).  The wrappers are exercised once, for the record.
+    L = swc_hip.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    conv_fn = L.swc_winograd2x2_conv if args.precision == "fp32" else L.swc_winograd2x2_conv_bf16
+    xp, wp, tip, yp = x.data_ptr(), w.data_ptr(), ti.data_ptr(), y.data_ptr()
+    winograd2x2_imTrans(x, relu=True, out=ti)
+    winograd2x2_conv(ti, w, precision=args.precision, out=y)
+
+    def f_imtrans():
+        if L.swc_winograd2x2_imtrans(xp, tip, C, B, H, W, 1, 1, 1, stream) != 0:
+            raise RuntimeError("swc_winograd2x2_imtrans failed")
+
+    def f_conv():
+        if conv_fn(tip, wp, yp, None, None, C, B, nH, nW, K, 1, 1, stream) != 0:
+            raise RuntimeError("swc_winograd2x2_conv failed")
+
+    def step():
+        f_imtrans()
+        f_conv()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # Per-kernel average launch durations, HIP events on the launching (current) stream.
+    ms_imtrans = time_loop(f_imtrans, args.steps, torch)
+    ms_conv = time_loop(f_conv, args.steps, torch)
+    ms_pair = time_loop(step, args.steps, torch)
+    torch.cuda.synchronize()
+
+    direct_flops = 18.0 * B * H * W * C * K
+    gemm_flops = 32.0 * M * C * K
+    imtrans_bytes = 4.0 * B * H * W * C + 64.0 * M * C
+    conv_bytes = 64.0 * M * C + 64.0 * C * K + 16.0 * M * K
+    tf_conv = gemm_flops / (ms_conv * 1e-3) / 1e12
+    gbs_imtrans = imtrans_bytes / (ms_imtrans * 1e-3) / 1e9
+    peak_tf = FP32_MFMA_PEAK_TF if args.precision == "fp32" else BF16_MFMA_PEAK_TF
+
+    out = {
+        "metric": "effective conv GFLOP/s + imTrans HBM GB/s, ResNet-18 conv3 batch 64, 1 MI355X",
+        "value": round(direct_flops / (ms_step * 1e-3) / 1e9, 1),
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if args.precision == "fp32" else "bf16 operands, f32 accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: winograd2x2_imTrans(+ReLU) + winograd2x2_conv, N=%d %dx%dx%d -> %d, fp32 NHWC, "
+                        "weights [16,%d,%d] at %.0f%% density" % (name, B, H, W, C, K, C, K, density * 100),
+            "tiles_M": M,
+            "input": kind,
+            "gemm_precision": args.precision,
+        },
+        "imtrans_GBps": round(gbs_imtrans, 1),
+        "conv_TFLOPs": round(tf_conv, 2),
+        "ms_imtrans": round(ms_imtrans, 5),
+        "ms_conv": round(ms_conv, 5),
+        "ms_pair_events": round(ms_pair, 5),
+        "roofline": {
+            "kernel": "winograd2x2_conv (16 GEMMs + fused A^T m A), %s" % args.precision,
+            "bound": "mfma",
+            "achieved": round(tf_conv, 2),
+            "peak": peak_tf,
+            "unit": "TFLOP/s",
+            "frac": round(tf_conv / peak_tf, 4),
+            "traffic": None,
+            "algorithmic_flop_per_launch": gemm_flops,
+            "algorithmic_bytes_per_launch": conv_bytes,
+        },
+        "roofline_imtrans": {
+            "kernel": "winograd2x2_imTrans + ReLU",
+            "bound": "hbm",
+            "achieved": round(gbs_imtrans, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(gbs_imtrans / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "algorithmic_bytes_per_launch": imtrans_bytes,
+        },
+    }
+
+    if not args.no_cpu:
+        cpu, ti_ref, y32_ref = cpu_baseline(name, x_np, w_np, args.cpu_budget)
+        out["cpu_baseline"] = cpu
+        # Parity gate on the very buffers that were timed.
+        import oracle
+        ti_gpu = ti.cpu().numpy()
+        y_gpu = y.cpu().numpy()
+        y_ref = oracle.conv(ti_ref, w_np, acc64=True)
+        den = float(np.max(np.abs(y_ref)))
+        out["parity"] = {
+            "imtrans_bit_exact": bool(np.array_equal(ti_gpu, ti_ref)),
+            "relu_zero_mask_equal": bool(np.array_equal(ti_gpu == 0, ti_ref == 0)),
+            "conv_max_rel_err": float(np.max(np.abs(y_gpu - y_ref)) / den),
+            "conv_l1_rel_err": float(np.sum(np.abs(y_gpu - y_ref)) / (np.sum(np.abs(y_gpu)) + np.sum(np.abs(y_ref)))),
+            "cpu_fp32_oracle_max_rel_err": float(np.max(np.abs(y32_ref - y_ref)) / den),
+        }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

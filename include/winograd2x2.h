@@ -1,0 +1,151 @@
+/*
+ * C ABI of the MI355X (gfx950) Winograd F(2x2,3x3) forward ops.
+ *
+ * Plain pointers and sizes only.  Every device pointer is owned by the caller; no
+ * entry point allocates or frees device memory, keeps state between calls, or
+ * synchronises: work is queued on `stream` (a hipStream_t passed as void*; NULL is
+ * the null stream) and the call returns.  Calls are re-entrant and thread-safe.
+ *
+ * Citations name the interface of the reference (xingyul/sparse-winograd-cnn) that
+ * each entry point stands in for; paths are relative to the reference checkout.
+ */
+#ifndef WINOGRAD2X2_H_
+#define WINOGRAD2X2_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *swc_stream_t;
+
+/* Exported from the shared library; everything else in it is hidden. */
+#define SWC_API __attribute__((visibility("default")))
+
+/* Status codes: 0 on success, negative on error.  Nothing here calls exit(). */
+#define SWC_OK 0
+#define SWC_ERR_NULL_POINTER (-1) /* a required pointer is NULL */
+#define SWC_ERR_BAD_DIMS (-2)     /* a dimension is <= 0, inconsistent, or too large to index */
+#define SWC_ERR_BAD_PAD (-3)      /* pad_h/pad_w other than 1: the only geometry the ops define */
+#define SWC_ERR_HIP (-4)          /* the HIP runtime refused the launch; see swc_last_hip_error() */
+#define SWC_ERR_BAD_RANK (-5)     /* op-level wrappers: wrong tensor rank or leading dimension */
+
+SWC_API const char *swc_strerror(int status);
+/* hipError_t of the most recent failed launch on the calling thread (0 if none). */
+SWC_API int swc_last_hip_error(void);
+/* Library version, "major.minor". */
+SWC_API const char *swc_version(void);
+
+/* ---------------------------------------------------------------------------
+ * Launcher level: what the reference's TensorFlow op kernels call.
+ * ------------------------------------------------------------------------- */
+
+/*
+ * Input transform T = B^T d B over 4x4 tiles at stride 2, pad 1, optionally followed by
+ * the Winograd-domain ReLU.
+ *   Input   [B,H,W,C]            fp32, NHWC, contiguous
+ *   TransIm [16,B,nH,nW,C]       fp32, nH=(H+1)/2, nW=(W+1)/2
+ * Replaces  void Winograd2x2ImTransComputeLauncher(const float *Input, float *TransIm,
+ *           int C, int B, int H, int W, int pad_h, int pad_w)
+ *   declared winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans_op.cc:30,
+ *   defined  winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans_cuda.cu.cc:151-157,
+ *   called   winograd2x2_imTrans_op.cc:55 (always with pad 1,1).
+ * `relu` != 0 fuses the tf.nn.relu that the layer wrapper applies to the op's result
+ * (ResNet-18-var/winograd_imtrans.py:16-17): t > 0 ? t : 0.  The 16 sums keep the
+ * reference's left-to-right association (…_cuda.cu.cc:112-127), so values and zero
+ * masks are bit-identical to it.  Unlike the reference, C is not limited to 1024.
+ */
+SWC_API int swc_winograd2x2_imtrans(const float *Input, float *TransIm, int C, int B, int H, int W,
+                            int pad_h, int pad_w, int relu, swc_stream_t stream);
+
+/*
+ * The 16 per-position products TI[i] (MxC) . Weight[i] (CxK), M = B*nH*nW, followed by
+ * the output transform Y = A^T p A, in one kernel (fp32 MFMA, fp32 accumulate).
+ *   Input  [16,B,nH,nW,C]  fp32      Weight [16,C,K] fp32
+ *   Output [B,2nH,2nW,K]   fp32, NHWC, never cropped
+ * Replaces  void Winograd2x2ConvComputeLauncher(const float *Input, const float *Weight,
+ *           float *Output, float *tmp_data_buffer, const long long *tmp_ptr_buffer,
+ *           int C, int B, int nH, int nW, int K, int pad_h, int pad_w)
+ *   declared winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_op.cc:31,
+ *   defined  winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_cuda.cu.cc:65-93
+ *   (assign :55-61, cublasSgemmBatched :80-85, Output_transform :12-53,87-89),
+ *   called   winograd2x2_conv_op.cc:66.
+ * tmp_data_buffer (16*M*K floats there) and tmp_ptr_buffer (48 pointers there) are kept
+ * in the signature for call-site compatibility and ignored: pass NULL.  The products
+ * never leave registers.  Unlike the reference, K is not limited to 1024.
+ */
+SWC_API int swc_winograd2x2_conv(const float *Input, const float *Weight, float *Output,
+                         float *tmp_data_buffer, const long long *tmp_ptr_buffer,
+                         int C, int B, int nH, int nW, int K, int pad_h, int pad_w,
+                         swc_stream_t stream);
+
+/*
+ * Same contract as swc_winograd2x2_conv, with both GEMM operands rounded to bf16
+ * (round-to-nearest-even) on their way into the matrix cores; accumulation and the
+ * output transform stay fp32.  No counterpart in the reference (its GEMM is cuBLAS
+ * SGEMM, winograd2x2_conv_cuda.cu.cc:80-85); an opt-in speed/precision trade.
+ */
+SWC_API int swc_winograd2x2_conv_bf16(const float *Input, const float *Weight, float *Output,
+                              float *tmp_data_buffer, const long long *tmp_ptr_buffer,
+                              int C, int B, int nH, int nW, int K, int pad_h, int pad_w,
+                              swc_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Op level: what the reference's OpKernel::Compute and shape functions do on the
+ * host (read dims from the tensors, derive the output shape, call the launcher).
+ * Shapes are int64 arrays in the reference's dimension order.
+ * ------------------------------------------------------------------------- */
+
+/*
+ * Shape rule of Winograd2x2ImTrans: [B,H,W,C] -> [16,B,(H+1)/2,(W+1)/2,C].
+ * winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans.py:20-27 and
+ * winograd2x2_imTrans_op.cc:42-51.
+ */
+SWC_API int swc_winograd2x2_imtrans_op_shape(int in_rank, const int64_t *in_dims, int64_t out_dims[5]);
+
+/*
+ * Winograd2x2ImTransCudaOp::Compute (winograd2x2_imTrans_op.cc:36-56) with the output
+ * passed in instead of allocated: validates that out_dims is what the shape rule gives,
+ * then launches with pad 1,1.
+ */
+SWC_API int swc_winograd2x2_imtrans_op_compute(const float *input, int in_rank, const int64_t *in_dims,
+                                       float *output, int out_rank, const int64_t *out_dims,
+                                       int relu, swc_stream_t stream);
+
+/*
+ * Shape rule of Winograd2x2Conv: I [16,B,nH,nW,C], W [16,C,K] -> [B,2nH,2nW,K].
+ * winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv.py:19-29 and
+ * winograd2x2_conv_op.cc:45-53.  The reference checks ranks only; this also requires
+ * I.dim0 == W.dim0 == 16 and W.dim1 == C.
+ */
+SWC_API int swc_winograd2x2_conv_op_shape(int in_rank, const int64_t *in_dims, int w_rank, const int64_t *w_dims,
+                                  int64_t out_dims[4]);
+
+/*
+ * Winograd2x2ConvCudaOp::Compute (winograd2x2_conv_op.cc:37-67) with the output passed
+ * in; no temporaries are needed.  precision: 0 = fp32 MFMA, 1 = bf16 operands.
+ */
+SWC_API int swc_winograd2x2_conv_op_compute(const float *input, int in_rank, const int64_t *in_dims,
+                                    const float *weight, int w_rank, const int64_t *w_dims,
+                                    float *output, int out_rank, const int64_t *out_dims,
+                                    int precision, swc_stream_t stream);
+
+#ifdef __cplusplus
+} /* extern "C" */
+
+/*
+ * C++ linkage, exact reference signatures: an unmodified winograd2x2_imTrans_op.cc /
+ * winograd2x2_conv_op.cc (which declare these at :30 / :31 and call them at :55 / :66)
+ * links against this library in place of the CUDA objects.  They run on the null
+ * stream, as the reference launches do, apply no ReLU, and report errors on stderr
+ * because the signatures return void.
+ */
+SWC_API void Winograd2x2ImTransComputeLauncher(const float *Input, float *TransIm, int C, int B, int H, int W,
+                                       int pad_h, int pad_w);
+SWC_API void Winograd2x2ConvComputeLauncher(const float *Input, const float *Weight, float *Output,
+                                    float *tmp_data_buffer, const long long *tmp_ptr_buffer,
+                                    int C, int B, int nH, int nW, int K, int pad_h, int pad_w);
+#endif
+
+#endif /* WINOGRAD2X2_H_ */

@@ -1,0 +1,31 @@
+// Status strings, version and the per-thread record of the last HIP error.
+#include "swc_common.h"
+
+namespace swc {
+namespace {
+thread_local int g_last_hip_error = 0;
+}
+
+int note_hip_error(hipError_t e)
+{
+    g_last_hip_error = static_cast<int>(e);
+    return SWC_ERR_HIP;
+}
+}  // namespace swc
+
+extern "C" const char *swc_strerror(int status)
+{
+    switch (status) {
+        case SWC_OK: return "ok";
+        case SWC_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case SWC_ERR_BAD_DIMS: return "a dimension is non-positive, inconsistent or too large";
+        case SWC_ERR_BAD_PAD: return "pad_h and pad_w must both be 1";
+        case SWC_ERR_HIP: return "the HIP runtime refused the launch (see swc_last_hip_error)";
+        case SWC_ERR_BAD_RANK: return "wrong tensor rank or leading dimension";
+        default: return "unknown status";
+    }
+}
+
+extern "C" int swc_last_hip_error(void) { return swc::g_last_hip_error; }
+
+extern "C" const char *swc_version(void) { return "0.1"; }

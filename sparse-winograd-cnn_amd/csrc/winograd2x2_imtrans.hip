@@ -1,0 +1,159 @@
+// Winograd F(2x2,3x3) input transform T = B^T d B with the Winograd-domain ReLU fused,
+// for gfx950.  NHWC [B,H,W,C] -> [16,B,nH,nW,C], 4x4 tiles at stride 2, pad 1.
+//
+// Stands in for Winograd2x2ImTransCompute / Winograd2x2ImTransComputeLauncher of the
+// reference (winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans_cuda.cu.cc:11-157)
+// plus the tf.nn.relu its layer wrapper applies afterwards
+// (ResNet-18-var/winograd_imtrans.py:16-17).
+//
+// The kernel is a pure stream: 4 bytes read and 64 bytes written per (tile, channel)
+// with 48 adds, so HBM bandwidth bounds it.  Channels are the contiguous axis, a lane
+// owns VEC consecutive channels and never needs another lane's data.
+
+#include "swc_common.h"
+
+namespace swc {
+namespace {
+
+// The 16 sums, each left to right in fp32, exactly as the reference writes them
+// (winograd2x2_imTrans_cuda.cu.cc:112-127).  There are no multiplies, hence nothing
+// for the compiler to contract, and fp adds are not reassociated without fast-math:
+// results are bit-identical to the reference's.
+__device__ __forceinline__ void bt_d_b(const float (&d)[16], float (&t)[16])
+{
+    t[0]  = d[0] - d[2] - d[8] + d[10];
+    t[1]  = d[1] + d[2] - d[9] - d[10];
+    t[2]  = d[2] - d[1] + d[9] - d[10];
+    t[3]  = d[1] - d[3] - d[9] + d[11];
+    t[4]  = d[4] - d[6] + d[8] - d[10];
+    t[5]  = d[5] + d[6] + d[9] + d[10];
+    t[6]  = d[6] - d[5] - d[9] + d[10];
+    t[7]  = d[5] - d[7] + d[9] - d[11];
+    t[8]  = d[6] - d[4] + d[8] - d[10];
+    t[9]  = d[9] - d[6] - d[5] + d[10];
+    t[10] = d[5] - d[6] - d[9] + d[10];
+    t[11] = d[7] - d[5] + d[9] - d[11];
+    t[12] = d[4] - d[6] - d[12] + d[14];
+    t[13] = d[5] + d[6] - d[13] - d[14];
+    t[14] = d[6] - d[5] + d[13] - d[14];
+    t[15] = d[5] - d[7] - d[13] + d[15];
+}
+
+template <int VEC>
+struct Vec;
+template <>
+struct Vec<1> {
+    using type = float;
+    static __device__ __forceinline__ float get(const float &v, int) { return v; }
+    static __device__ __forceinline__ void set(float &v, int, float x) { v = x; }
+    static __device__ __forceinline__ float zero() { return 0.0f; }
+};
+template <>
+struct Vec<4> {
+    using type = float4;
+    static __device__ __forceinline__ float get(const float4 &v, int q)
+    {
+        return q == 0 ? v.x : q == 1 ? v.y : q == 2 ? v.z : v.w;
+    }
+    static __device__ __forceinline__ void set(float4 &v, int q, float x)
+    {
+        if (q == 0) v.x = x; else if (q == 1) v.y = x; else if (q == 2) v.z = x; else v.w = x;
+    }
+    static __device__ __forceinline__ float4 zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+};
+
+template <int VEC, bool RELU>
+__device__ __forceinline__ void transform_vec(const typename Vec<VEC>::type (&d)[16], typename Vec<VEC>::type (&t)[16])
+{
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) {
+        float ds[16], ts[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) ds[j] = Vec<VEC>::get(d[j], q);
+        bt_d_b(ds, ts);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float v = ts[i];
+            if (RELU) v = v > 0.0f ? v : 0.0f;
+            Vec<VEC>::set(t[i], q, v);
+        }
+    }
+}
+
+// One lane per (tile, channel vector).  Lanes are numbered along the flattened
+// [M, C/VEC] plane of the output, so each of the 16 stores of a wavefront covers
+// 64*VEC*4 contiguous bytes of one plane whatever C is; the 16 loads of a wavefront
+// are contiguous per tile and overlap between neighbouring tiles in L1/L2.
+template <int VEC, bool RELU, typename Idx>
+__global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__restrict__ X, float *__restrict__ TI,
+                                                             int H, int W, int C, int nH, int nW, Idx items,
+                                                             size_t plane)
+{
+    using V = typename Vec<VEC>::type;
+    const Idx idx = static_cast<Idx>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= items) return;
+    const int CV = C / VEC;
+    const int cv = static_cast<int>(idx % CV);
+    Idx m = idx / CV;
+    const int tw = static_cast<int>(m % nW);
+    m /= nW;
+    const int th = static_cast<int>(m % nH);
+    const size_t b = static_cast<size_t>(m / nH);
+
+    const int y0 = 2 * th - 1, x0 = 2 * tw - 1;
+    const float *img = X + b * H * W * C + static_cast<size_t>(cv) * VEC;
+    V d[16];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int y = y0 + r;
+        const bool yin = (y > -1) && (y < H);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int x = x0 + s;
+            const bool in = yin && (x > -1) && (x < W);
+            d[4 * r + s] = in ? *reinterpret_cast<const V *>(img + (static_cast<size_t>(y) * W + x) * C)
+                              : Vec<VEC>::zero();
+        }
+    }
+    V t[16];
+    transform_vec<VEC, RELU>(d, t);
+    float *dst = TI + static_cast<size_t>(idx) * VEC;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) *reinterpret_cast<V *>(dst + i * plane) = t[i];
+}
+
+template <int VEC, bool RELU, typename Idx>
+int launch_direct(const float *X, float *TI, int B, int H, int W, int C, int nH, int nW, hipStream_t stream)
+{
+    const size_t M = static_cast<size_t>(B) * nH * nW;
+    const size_t items = M * (C / VEC);
+    const size_t blocks = (items + 255) / 256;
+    imtrans_direct_kernel<VEC, RELU, Idx><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(
+        X, TI, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
+    return check_launch();
+}
+
+}  // namespace
+}  // namespace swc
+
+extern "C" int swc_winograd2x2_imtrans(const float *Input, float *TransIm, int C, int B, int H, int W,
+                                       int pad_h, int pad_w, int relu, swc_stream_t stream)
+{
+    using namespace swc;
+    if (Input == nullptr || TransIm == nullptr) return SWC_ERR_NULL_POINTER;
+    if (C <= 0 || B <= 0 || H <= 0 || W <= 0) return SWC_ERR_BAD_DIMS;
+    if (pad_h != 1 || pad_w != 1) return SWC_ERR_BAD_PAD;
+    const int nH = (H + 1) / 2, nW = (W + 1) / 2;
+    const size_t M = static_cast<size_t>(B) * nH * nW;
+    // One lane per item, 256 per workgroup, grid.x below 2^31.
+    if (M * C / 256 >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool vec = (C % 4 == 0) && aligned16(Input) && aligned16(TransIm);
+    const bool small = M * C < (1ull << 31);
+#define SWC_DISPATCH(VEC, RELU)                                                           \
+    (small ? launch_direct<VEC, RELU, unsigned>(Input, TransIm, B, H, W, C, nH, nW, s)    \
+           : launch_direct<VEC, RELU, unsigned long long>(Input, TransIm, B, H, W, C, nH, nW, s))
+    if (vec) return relu ? SWC_DISPATCH(4, true) : SWC_DISPATCH(4, false);
+    return relu ? SWC_DISPATCH(1, true) : SWC_DISPATCH(1, false);
+#undef SWC_DISPATCH
+}

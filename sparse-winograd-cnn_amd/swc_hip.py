@@ -1,0 +1,110 @@
+"""ctypes binding of libwinograd2x2_hip.so (the C ABI declared in include/winograd2x2.h).
+
+There is no fallback: if the library has not been built, loading raises.
+"""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libwinograd2x2_hip.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+SWC_OK = 0
+SWC_ERR_NULL_POINTER = -1
+SWC_ERR_BAD_DIMS = -2
+SWC_ERR_BAD_PAD = -3
+SWC_ERR_HIP = -4
+SWC_ERR_BAD_RANK = -5
+
+# Every symbol include/winograd2x2.h declares with C linkage.
+C_SYMBOLS = (
+    "swc_strerror", "swc_last_hip_error", "swc_version",
+    "swc_winograd2x2_imtrans", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
+    "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
+    "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
+)
+# The two C++-linkage launchers with the reference's exact signatures (Itanium mangling).
+CXX_SYMBOLS = (
+    "_Z33Winograd2x2ImTransComputeLauncherPKfPfiiiiii",
+    "_Z30Winograd2x2ConvComputeLauncherPKfS0_PfS1_PKxiiiiiii",
+)
+
+_lib = None
+
+
+def build():
+    """Compile the library for gfx950 with hipcc (works without a GPU)."""
+    subprocess.check_call(["make", "-s", "-C", CSRC, "-j8"])
+    return LIB_PATH
+
+
+class SwcError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        msg = lib().swc_strerror(status).decode()
+        if status == SWC_ERR_HIP:
+            msg += " [hipError_t %d]" % lib().swc_last_hip_error()
+        super().__init__("%s: %s (status %d)" % (where, msg, status))
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                "%s is missing: build it with `make -C %s` (or __graft_entry__.build()); "
+                "there is no CPU or PyTorch fallback for these ops" % (LIB_PATH, CSRC))
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i32, fp = ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p
+        i64p = ctypes.POINTER(ctypes.c_int64)
+        L.swc_strerror.restype = ctypes.c_char_p
+        L.swc_strerror.argtypes = [i32]
+        L.swc_last_hip_error.restype = i32
+        L.swc_last_hip_error.argtypes = []
+        L.swc_version.restype = ctypes.c_char_p
+        L.swc_version.argtypes = []
+        L.swc_winograd2x2_imtrans.restype = i32
+        L.swc_winograd2x2_imtrans.argtypes = [fp, fp] + [i32] * 7 + [vp]
+        for f in (L.swc_winograd2x2_conv, L.swc_winograd2x2_conv_bf16):
+            f.restype = i32
+            f.argtypes = [fp, fp, fp, fp, vp] + [i32] * 7 + [vp]
+        L.swc_winograd2x2_imtrans_op_shape.restype = i32
+        L.swc_winograd2x2_imtrans_op_shape.argtypes = [i32, i64p, i64p]
+        L.swc_winograd2x2_imtrans_op_compute.restype = i32
+        L.swc_winograd2x2_imtrans_op_compute.argtypes = [fp, i32, i64p, fp, i32, i64p, i32, vp]
+        L.swc_winograd2x2_conv_op_shape.restype = i32
+        L.swc_winograd2x2_conv_op_shape.argtypes = [i32, i64p, i32, i64p, i64p]
+        L.swc_winograd2x2_conv_op_compute.restype = i32
+        L.swc_winograd2x2_conv_op_compute.argtypes = [fp, i32, i64p, fp, i32, i64p, fp, i32, i64p, i32, vp]
+        _lib = L
+    return _lib
+
+
+def dims(shape):
+    return (ctypes.c_int64 * len(shape))(*[int(s) for s in shape])
+
+
+def check(status, where):
+    if status != SWC_OK:
+        raise SwcError(status, where)
+
+
+def require_cuda_f32(t, name, rank):
+    """The checks a TensorFlow kernel registration did implicitly (float, DEVICE_GPU)."""
+    import torch
+
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("%s must be a torch.Tensor, got %s" % (name, type(t).__name__))
+    if t.dim() != rank:
+        raise ValueError("%s must have rank %d, got shape %s" % (name, rank, tuple(t.shape)))
+    if t.dtype != torch.float32:
+        raise TypeError("%s must be float32, got %s" % (name, t.dtype))
+    if not t.is_cuda:
+        # The reference's CPU kernels print a message and exit(-1)
+        # (winograd2x2_imTrans_op.cc:82-83, winograd2x2_conv_op.cc:89-90); here it is an error.
+        raise RuntimeError("%s is on %s: these ops run on the GPU only (no CPU kernel exists)" % (name, t.device))
+    if torch.is_grad_enabled() and t.requires_grad:
+        raise NotImplementedError(
+            "%s requires grad: only the forward ops are implemented; wrap the call in torch.no_grad()" % name)
+    return t.contiguous()

@@ -1,0 +1,49 @@
+"""Python binding of the Winograd2x2Conv op for PyTorch-ROCm tensors.
+
+Mirrors winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv.py of the reference:
+``winograd2x2_conv(I, W)`` (:13-14) with the shape rule of its RegisterShape function
+(:19-29).  The gradient registration (:31-36) has no counterpart: forward only.
+"""
+import os
+import sys
+
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+import swc_hip  # noqa: E402
+
+PRECISIONS = {"fp32": 0, "bf16": 1}
+
+
+def winograd2x2_conv_shape(i_shape, w_shape):
+    """I [16,B,nH,nW,C], W [16,C,K] -> [B,2nH,2nW,K] (winograd2x2_conv.py:19-29), computed by the C++ host wrapper."""
+    out = swc_hip.dims([0] * 4)
+    swc_hip.check(swc_hip.lib().swc_winograd2x2_conv_op_shape(
+        len(i_shape), swc_hip.dims(i_shape), len(w_shape), swc_hip.dims(w_shape), out), "winograd2x2_conv")
+    return tuple(out)
+
+
+def winograd2x2_conv(I, W, precision="fp32", out=None):
+    """I: [16,B,nH,nW,C], W: [16,C,K], float32 on the GPU -> [B,2nH,2nW,K] (uncropped).
+
+    ``precision="bf16"`` rounds both GEMM operands to bf16 (fp32 accumulate).
+    """
+    if precision not in PRECISIONS:
+        raise ValueError("precision must be one of %s" % sorted(PRECISIONS))
+    I = swc_hip.require_cuda_f32(I, "I", 5)
+    W = swc_hip.require_cuda_f32(W, "W", 3)
+    if W.device != I.device:
+        raise ValueError("I and W must be on the same device")
+    shape = winograd2x2_conv_shape(I.shape, W.shape)
+    if out is None:
+        out = torch.empty(shape, dtype=torch.float32, device=I.device)
+    else:
+        if tuple(out.shape) != shape or out.dtype != torch.float32 or out.device != I.device or not out.is_contiguous():
+            raise ValueError("out must be a contiguous float32 tensor of shape %s on %s" % (shape, I.device))
+    with torch.cuda.device(I.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        st = swc_hip.lib().swc_winograd2x2_conv_op_compute(
+            I.data_ptr(), 5, swc_hip.dims(I.shape), W.data_ptr(), 3, swc_hip.dims(W.shape),
+            out.data_ptr(), 4, swc_hip.dims(out.shape), PRECISIONS[precision], stream)
+    swc_hip.check(st, "winograd2x2_conv")
+    return out

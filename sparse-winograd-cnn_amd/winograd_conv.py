@@ -1,0 +1,61 @@
+"""Layer wrapper WinogradConv, after ResNet-18-var/winograd_conv.py:15-28."""
+import math
+import os
+import sys
+
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+import winograd2x2_conv.winograd2x2_conv  # noqa: E402
+
+__all__ = ["WinogradConv"]
+
+
+class WinogradConv(torch.nn.Module):
+    """Holds the Winograd-domain weights W [16, in_channel, out_channel] and applies the op.
+
+    Arguments follow ``WinogradConv(x, in_channel, out_channel, mask=None, W_init=None)``
+    of the reference (winograd_conv.py:16), with ``x`` moved to ``forward``:
+
+    * ``W_init``: callable filling a tensor in place, or a tensor/array of the weight's
+      shape.  Default: the reference's ``variance_scaling_initializer(factor=2*9/32)``
+      (:18-19): a normal truncated at two standard deviations with
+      std = sqrt(1.3*factor/fan_in), fan_in = 16*in_channel as TensorFlow 1.x computes
+      it for a rank-3 shape.
+    * ``mask``: optional 0/1 array of the weight's shape; the reference multiplies it in on
+      every step (:23-25).  Here the product W*mask is cached and refreshed by
+      ``refresh()`` after W changes.
+
+    Forward only: W carries no gradient.
+    """
+
+    def __init__(self, in_channel, out_channel, mask=None, W_init=None, precision="fp32", device=None):
+        super().__init__()
+        self.in_channel, self.out_channel, self.precision = int(in_channel), int(out_channel), precision
+        W = torch.empty(16, self.in_channel, self.out_channel, dtype=torch.float32, device=device)
+        if W_init is None:
+            std = math.sqrt(1.3 * (2.0 * 9.0 / 32.0) / (16 * self.in_channel))
+            torch.nn.init.trunc_normal_(W, mean=0.0, std=std, a=-2 * std, b=2 * std)
+        elif callable(W_init):
+            W_init(W)
+        else:
+            W.copy_(torch.as_tensor(W_init, dtype=torch.float32).reshape(W.shape))
+        self.W = torch.nn.Parameter(W, requires_grad=False)
+        if mask is not None:
+            mask = torch.as_tensor(mask, dtype=torch.float32, device=W.device).reshape(W.shape).clone()
+        self.register_buffer("mask", mask)
+        self._masked = None
+
+    def refresh(self):
+        """Recompute the cached W*mask (call after changing W or mask)."""
+        self._masked = None
+
+    def masked_weight(self):
+        if self.mask is None:
+            return self.W.data
+        if self._masked is None or self._masked.device != self.W.device:
+            self._masked = (self.W.data * self.mask).contiguous()
+        return self._masked
+
+    def forward(self, x):
+        return winograd2x2_conv.winograd2x2_conv.winograd2x2_conv(x, self.masked_weight(), precision=self.precision)
