@@ -1,0 +1,621 @@
+// The fused GEMM + output-transform kernel of the Winograd convolution (device code).
+// See winograd2x2_conv.hip for what it replaces in the reference.
+#pragma once
+
+#include "swc_common.h"
+
+namespace swc {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+
+// Signs of A^T (x) A^T: bit (4*i + j) set when +-P_i enters Y_j, j = 2*dy + dx.
+// Row i = 4r+s contributes AT[dy][r]*AT[dx][s] with AT = [[1,1,1,0],[0,1,-1,-1]]
+// (the sums at winograd2x2_conv_cuda.cu.cc:39-46).
+constexpr int kAT[2][4] = {{1, 1, 1, 0}, {0, 1, -1, -1}};
+constexpr unsigned long long sign_mask(int want)
+{
+    unsigned long long m = 0;
+    for (int i = 0; i < 16; ++i)
+        for (int j = 0; j < 4; ++j)
+            if (kAT[j / 2][i / 4] * kAT[j % 2][i % 4] == want) m |= 1ull << (4 * i + j);
+    return m;
+}
+constexpr unsigned long long kPlus = sign_mask(1);
+constexpr unsigned long long kMinus = sign_mask(-1);
+
+// Round an fp32 value to the nearest bf16 (ties to even) and return it widened back to fp32.
+__device__ __forceinline__ float round_bf16(float x)
+{
+    unsigned u = __float_as_uint(x);
+    if ((u & 0x7f800000u) == 0x7f800000u) return x;  // inf / nan pass through
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return __uint_as_float(u & 0xffff0000u);
+}
+
+__device__ __forceinline__ float4 round_bf16(float4 v)
+{
+    return make_float4(round_bf16(v.x), round_bf16(v.y), round_bf16(v.z), round_bf16(v.w));
+}
+
+// Buffer descriptor over [base, base+bytes): loads through it return 0 beyond the end.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, unsigned bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+__device__ __forceinline__ float4 buffer_load_f4(__amdgpu_buffer_rsrc_t r, unsigned byte_offset)
+{
+    return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(byte_offset), 0, 0));
+}
+
+constexpr unsigned kOutOfRange = 0xfffffff0u;  // a byte offset no descriptor here reaches
+
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int OCC_ = 2>
+struct ConvCfg {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
+    static constexpr int OCC = OCC_;                     // waves per SIMD the register budget allows
+    static constexpr int NT = WGM * WGN * 64;            // threads per workgroup
+    static constexpr int WM = BM / WGM, WN = BN / WGN;   // wave tile
+    static constexpr int TM = WM / 32, TN = WN / 32;     // 32x32 MFMA tiles per wave
+    static constexpr int LDA = BK + 4;  // row stride (floats): 4*odd keeps b128 row reads conflict-free
+    static constexpr int LDB = BN + 4;
+    static constexpr int NA = BM * BK / (4 * NT);        // float4 per thread per A tile
+    static constexpr int NB = BK * BN / (4 * NT);
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile is made of 32x32 MFMA tiles");
+    static_assert(BK % 8 == 0, "a k-step feeds 4 MFMAs from one b128 read per lane group");
+    static_assert((BK / 4) % 2 == 1 || BK % 8 == 0, "LDA");
+    static_assert(BM * BK % (4 * NT) == 0 && BK * BN % (4 * NT) == 0, "tile loads divide evenly");
+};
+
+// Scatter of the four output tiles: tile row m = (b*nH + th)*nW + tw -> pixels (2th+dy, 2tw+dx)
+// of image b (winograd2x2_conv_cuda.cu.cc:48-51).  Accumulator register r of lane (lg, li)
+// holds row 8*(r/4) + 4*lg + r%4 and column li of a 32x32 tile.  M < 2^31 (checked by the
+// launcher), so tile-row arithmetic fits 32 bits.
+template <typename Cfg>
+__device__ __forceinline__ void store_output(const floatx16 (&Y)[4][Cfg::TM][Cfg::TN], float *__restrict__ Out,
+                                             size_t M, int K, int nW, size_t m0, int n0, int wm0, int wn0, int li,
+                                             int lg)
+{
+    constexpr int TM = Cfg::TM, TN = Cfg::TN;
+    const size_t oW = 2 * static_cast<size_t>(nW);
+    const size_t row_stride = oW * K;
+    const unsigned M32 = static_cast<unsigned>(M), m032 = static_cast<unsigned>(m0);
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const unsigned gm = m032 + wm0 + tm * 32 + 8 * (r / 4) + 4 * lg + (r % 4);
+            if (gm >= M32) continue;
+            const unsigned bt = gm / static_cast<unsigned>(nW);  // b*nH + th
+            const unsigned tw = gm - bt * static_cast<unsigned>(nW);
+            float *o = Out + (static_cast<size_t>(bt) * 2 * oW + 2 * tw) * K;
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) {
+                const int col = n0 + wn0 + tn * 32 + li;
+                if (col >= K) continue;
+                o[col] = Y[0][tm][tn][r];
+                o[K + col] = Y[1][tm][tn][r];
+                o[row_stride + col] = Y[2][tm][tn][r];
+                o[row_stride + K + col] = Y[3][tm][tn][r];
+            }
+        }
+    }
+}
+
+// FAST: C and K are multiples of 4, TI and Wt 16-byte aligned, and a tile's rows fit 32-bit
+//       byte offsets: global loads go through buffer descriptors, 16 bytes per lane, with the
+//       ragged edges (rows beyond M, channels beyond C, columns beyond K) returned as zeros by
+//       the descriptor's range check instead of by branches.
+//       Otherwise: scalar, individually guarded loads (any C, K and alignment).
+// BF16: both operands are rounded to bf16 on their way into LDS.
+template <typename Cfg, bool FAST, bool BF16>
+__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_mfma_kernel(
+    const float *__restrict__ TI, const float *__restrict__ Wt, float *__restrict__ Out, size_t M, int C, int K, int nH,
+    int nW, unsigned tiles_n)
+{
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, LDA = Cfg::LDA, LDB = Cfg::LDB, NA = Cfg::NA, NB = Cfg::NB;
+    constexpr int KS = BK / 8;
+
+    __shared__ __attribute__((aligned(16))) float As[2][BM * LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
+
+    const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
+    const size_t m0 = static_cast<size_t>(lid / tiles_n) * BM;
+    const int n0 = static_cast<int>(lid % tiles_n) * BN;
+    const unsigned rows_valid = static_cast<unsigned>(M - m0 < BM ? M - m0 : BM);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 31, lg = lane >> 5;
+    const int wm0 = (wave / Cfg::WGN) * Cfg::WM, wn0 = (wave % Cfg::WGN) * Cfg::WN;
+
+    // Per-thread constants of the tile loads: element f = tid + q*NT of a tile.
+    unsigned a_voff[NA], b_voff[NB];  // byte offsets within the tile's descriptor (FAST)
+    int a_cl[NA];                     // channel within the BK chunk
+#pragma unroll
+    for (int q = 0; q < NA; ++q) {
+        const int f = tid + q * NT;
+        a_cl[q] = (f % (BK / 4)) * 4;
+        a_voff[q] = (static_cast<unsigned>(f / (BK / 4)) * C + a_cl[q]) * 4u;
+    }
+#pragma unroll
+    for (int q = 0; q < NB; ++q) {
+        const int f = tid + q * NT;
+        const int n = n0 + (f % (BN / 4)) * 4;
+        b_voff[q] = n < K ? (static_cast<unsigned>(f / (BN / 4)) * K + n) * 4u : kOutOfRange;
+    }
+
+    float4 ra[NA], rb[NB];
+
+    // Fetch the tiles of (position pos, channels c0 .. c0+BK) into registers.
+    auto load_global = [&](int pos, int c0) {
+        if (FAST) {
+            // Descriptors start at the tile's first element of this chunk and end with the tile's
+            // last valid row (A) / the last channel row (B), so rows past either read as zero.
+            const float *a_base = TI + (static_cast<size_t>(pos) * M + m0) * C + c0;
+            const float *b_base = Wt + (static_cast<size_t>(pos) * C + c0) * K;
+            const __amdgpu_buffer_rsrc_t ra_desc = make_rsrc(a_base, (rows_valid * static_cast<unsigned>(C) - c0) * 4u);
+            const __amdgpu_buffer_rsrc_t rb_desc = make_rsrc(b_base, static_cast<unsigned>(C - c0) * K * 4u);
+#pragma unroll
+            for (int q = 0; q < NA; ++q)
+                ra[q] = buffer_load_f4(ra_desc, c0 + a_cl[q] < C ? a_voff[q] : kOutOfRange);
+#pragma unroll
+            for (int q = 0; q < NB; ++q) rb[q] = buffer_load_f4(rb_desc, b_voff[q]);
+        } else {
+            const float *a_base = TI + static_cast<size_t>(pos) * M * C;
+            const float *b_base = Wt + static_cast<size_t>(pos) * C * K;
+#pragma unroll
+            for (int q = 0; q < NA; ++q) {
+                const int f = tid + q * NT;
+                const int c = c0 + a_cl[q];
+                const size_t gm = m0 + f / (BK / 4);
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (gm < M) {
+                    const float *p = a_base + gm * C + c;
+                    if (c + 0 < C) v.x = p[0];
+                    if (c + 1 < C) v.y = p[1];
+                    if (c + 2 < C) v.z = p[2];
+                    if (c + 3 < C) v.w = p[3];
+                }
+                ra[q] = v;
+            }
+#pragma unroll
+            for (int q = 0; q < NB; ++q) {
+                const int f = tid + q * NT;
+                const int n = n0 + (f % (BN / 4)) * 4;
+                const int c = c0 + f / (BN / 4);
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (c < C) {
+                    const float *p = b_base + static_cast<size_t>(c) * K + n;
+                    if (n + 0 < K) v.x = p[0];
+                    if (n + 1 < K) v.y = p[1];
+                    if (n + 2 < K) v.z = p[2];
+                    if (n + 3 < K) v.w = p[3];
+                }
+                rb[q] = v;
+            }
+        }
+    };
+
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < NA; ++q) {
+            const int f = tid + q * NT;
+            *reinterpret_cast<float4 *>(&As[buf][(f / (BK / 4)) * LDA + (f % (BK / 4)) * 4]) =
+                BF16 ? round_bf16(ra[q]) : ra[q];
+        }
+#pragma unroll
+        for (int q = 0; q < NB; ++q) {
+            const int f = tid + q * NT;
+            *reinterpret_cast<float4 *>(&Bs[buf][(f / (BN / 4)) * LDB + (f % (BN / 4)) * 4]) =
+                BF16 ? round_bf16(rb[q]) : rb[q];
+        }
+    };
+
+    floatx16 Y[4][TM][TN];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) Y[j][tm][tn][r] = 0.f;
+
+    load_global(0, 0);
+    store_lds(0);
+    __syncthreads();
+
+    // (position, channel chunk) of the next tile to fetch, and the LDS buffer being read.
+    int npos = 0, nc0 = 0, buf = 0;
+
+    // The position loop is fully unrolled so that the signs of the output transform are
+    // compile-time constants; the loop over C stays a run-time loop.
+#pragma unroll
+    for (int pos = 0; pos < 16; ++pos) {
+        floatx16 P[TM][TN];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) P[tm][tn][r] = 0.f;
+
+        for (int c0 = 0; c0 < C; c0 += BK) {
+            nc0 += BK;
+            if (nc0 >= C) {
+                nc0 = 0;
+                ++npos;
+            }
+            const bool more = npos < 16;
+            if (more) load_global(npos, nc0);
+
+            const float *as = As[buf];
+            const float *bs = Bs[buf];
+            // All LDS reads of the step are issued before its first MFMA so that their latency
+            // overlaps the matrix pipeline.  Lane group lg feeds reduction indices
+            // k8*8+4*lg .. +3, one per MFMA; the order in which indices are reduced is free as
+            // long as A and B agree.
+            float4 a[KS][TM];
+            float b[KS][4][TN];
+#pragma unroll
+            for (int k8 = 0; k8 < KS; ++k8) {
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm)
+                    a[k8][tm] = *reinterpret_cast<const float4 *>(&as[(wm0 + tm * 32 + li) * LDA + k8 * 8 + 4 * lg]);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int tn = 0; tn < TN; ++tn)
+                        b[k8][t][tn] = bs[(k8 * 8 + 4 * lg + t) * LDB + wn0 + tn * 32 + li];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int k8 = 0; k8 < KS; ++k8)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int tm = 0; tm < TM; ++tm) {
+                        const float av = t == 0 ? a[k8][tm].x : t == 1 ? a[k8][tm].y : t == 2 ? a[k8][tm].z : a[k8][tm].w;
+#pragma unroll
+                        for (int tn = 0; tn < TN; ++tn)
+                            P[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b[k8][t][tn], P[tm][tn], 0, 0, 0);
+                    }
+            __builtin_amdgcn_sched_barrier(0);
+
+            if (more) store_lds(buf ^ 1);
+            __syncthreads();
+            buf ^= 1;
+        }
+
+        // P_pos is complete: fold it into the running output tiles, ascending pos.
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            constexpr unsigned long long plus = kPlus, minus = kMinus;
+            const int bit = 4 * pos + j;
+            if ((plus >> bit) & 1ull) {
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < TN; ++tn) Y[j][tm][tn] += P[tm][tn];
+            } else if ((minus >> bit) & 1ull) {
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < TN; ++tn) Y[j][tm][tn] -= P[tm][tn];
+            }
+        }
+        // Pin the updates here.  Y is not read again until the final stores, so without this the
+        // compiler defers all the adds to the end and keeps the 16 product tiles alive instead
+        // of the 4 running sums (4x the registers).
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn) asm volatile("" : "+v"(Y[j][tm][tn]));
+    }
+
+    store_output<Cfg>(Y, Out, M, K, nW, m0, n0, wm0, wn0, li, lg);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Asynchronous variant: tiles go from global memory straight into LDS (global_load_lds_dwordx4,
+// 16 bytes per lane, no VGPR staging and no ds_write), NSTAGE tiles deep, so that the
+// HBM/L2 latency of a tile is covered by the MFMA work of the NSTAGE-2 steps before it.
+//
+// Requirements checked by the launcher: C % BK == 0, K % 4 == 0, TI and Wt 16-byte aligned,
+// tile offsets below 2^31 bytes.  Rows beyond M and columns beyond K are not zero-filled but
+// clamped to the last valid row / column group: what they produce lands in accumulator rows
+// and columns that are never stored.
+//
+// LDS layout of one stage (floats):
+//   A: BM rows of BK/4 16-byte chunks; chunk j of row r sits in slot r*(BK/4) + (j ^ (r % (BK/4)))
+//      so that the 8 lanes served together by one ds_read_b128 cycle (8 consecutive rows, same
+//      chunk) fall into 8 different bank groups.  The swizzle is applied on the global side: a
+//      lane always writes LDS slot (wave-uniform base + lane), and picks the global chunk that
+//      belongs there.
+//   B: BK rows of BN floats, unswizzled (a wavefront reads 32 consecutive floats of a row).
+//
+// The loads are inline assembly on purpose: the compiler's wait-count insertion would otherwise
+// drain every outstanding load before each LDS read (it cannot tell the stages of the ring
+// apart).  Their completion is tracked by hand with s_waitcnt vmcnt(n); loads return in order.
+// ---------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ unsigned lds_address(const void *p)
+{
+    // generic -> LDS address space: the 32-bit value is the byte offset within the workgroup's LDS
+    return static_cast<unsigned>(reinterpret_cast<size_t>((const __attribute__((address_space(3))) char *)p));
+}
+
+// One 16-byte-per-lane global -> LDS copy: lane l reads base + voff (bytes) and writes LDS byte
+// address lds_base + 16*l.  lds_base must be wave-uniform.
+__device__ __forceinline__ void async_copy16(const float *base, unsigned voff, unsigned lds_base)
+{
+    asm volatile(
+        "s_mov_b32 m0, %2\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %1"
+        :
+        : "v"(voff), "s"(base), "s"(lds_base)
+        : "memory");  // m0 is a reserved register: the compiler never keeps a value in it across statements
+}
+
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding: vmcnt in bits 3:0
+// and 15:14, expcnt 6:4, lgkmcnt 11:8).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+    asm volatile("" ::: "memory");
+}
+
+template <typename Cfg, int NSTAGE>
+__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_mfma_async_kernel(
+    const float *__restrict__ TI, const float *__restrict__ Wt, float *__restrict__ Out, size_t M, int C, int K, int nH,
+    int nW, unsigned tiles_n)
+{
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, NA = Cfg::NA, NB = Cfg::NB;
+    constexpr int KS = BK / 8, CH = BK / 4, NWAVES = NT / 64;
+    constexpr int A_FLOATS = BM * BK, B_FLOATS = BK * BN, STAGE_FLOATS = A_FLOATS + B_FLOATS;
+    constexpr int LPS = NA + NB;  // loads per thread per step
+    static_assert(NSTAGE >= 2, "a ring needs two slots");
+    static_assert(KS % 2 == 0, "the MFMA chain of a step is split in two halves");
+    static_assert((CH & (CH - 1)) == 0, "swizzle needs a power-of-two chunk count");
+    static_assert(BM % (64 / CH) == 0 && (BM * CH) % 64 == 0 && (BK * BN / 4) % 64 == 0, "whole wave-loads");
+    static_assert((NSTAGE - 2) * LPS < 64, "vmcnt range");
+
+    __shared__ __attribute__((aligned(1024))) float smem[NSTAGE * STAGE_FLOATS];
+
+    const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
+    const size_t m0 = static_cast<size_t>(lid / tiles_n) * BM;
+    const int n0 = static_cast<int>(lid % tiles_n) * BN;
+    const unsigned rows_valid = static_cast<unsigned>(M - m0 < BM ? M - m0 : BM);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 31, lg = lane >> 5;
+    const int wm0 = (wave / Cfg::WGN) * Cfg::WM, wn0 = (wave % Cfg::WGN) * Cfg::WN;
+
+    // Per-thread byte offsets of the copies (constant over the whole kernel) and the
+    // wave-uniform LDS byte offsets, relative to a stage, they land at.
+    unsigned a_voff[NA], b_voff[NB];
+#pragma unroll
+    for (int q = 0; q < NA; ++q) {
+        const unsigned slot = (q * NWAVES + wave) * 64 + lane;
+        unsigned row = slot / CH;
+        const unsigned chunk = (slot % CH) ^ (row % CH);
+        row = row < rows_valid ? row : rows_valid - 1;
+        a_voff[q] = (row * static_cast<unsigned>(C) + chunk * 4) * 4u;
+    }
+#pragma unroll
+    for (int q = 0; q < NB; ++q) {
+        const unsigned slot = (q * NWAVES + wave) * 64 + lane;
+        const unsigned krow = slot / (BN / 4);
+        unsigned n = n0 + (slot % (BN / 4)) * 4;
+        n = n + 4 <= static_cast<unsigned>(K) ? n : static_cast<unsigned>(K) - 4;
+        b_voff[q] = (krow * static_cast<unsigned>(K) + n) * 4u;
+    }
+    const unsigned smem_base = lds_address(smem);
+    const unsigned wave_lds = __builtin_amdgcn_readfirstlane(wave) * 1024u;
+
+    const int nkc = C / BK;
+    floatx16 Y[4][TM][TN];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) Y[j][tm][tn][r] = 0.f;
+
+    // ---- copy issuer: running pointers to the tiles of the next step to fetch -------------
+    // Tile of (pos, c0): A at TI + (pos*M + m0)*C + c0, B at Wt + (pos*C + c0)*K.  Consecutive
+    // steps advance A by BK floats, plus (M-1)*C when the position wraps, and B by BK*K.
+    const float *a_next = TI + m0 * C;
+    const float *b_next = Wt;
+    const size_t a_wrap = (M - 1) * static_cast<size_t>(C);
+    const size_t b_inc = static_cast<size_t>(BK) * K;
+    int kc_next = 0, pos_next = 0;
+    unsigned lds_next = smem_base + wave_lds;  // this wave's first copy target in the next ring slot
+    int slot_next = 0;
+    auto copy = [&](int i) {  // the i-th of this thread's LPS copies of a step
+        if (i < NA)
+            async_copy16(a_next, a_voff[i < NA ? i : 0], lds_next + i * (NWAVES * 1024));
+        else
+            async_copy16(b_next, b_voff[i >= NA ? i - NA : 0], lds_next + A_FLOATS * 4 + (i - NA) * (NWAVES * 1024));
+    };
+    // After the last step the issuer wraps around to the first tile again: the loop below
+    // issues one step's copies per step unconditionally (so the outstanding-copy count is the
+    // same at every wait), and the surplus copies at the end re-fetch valid memory into ring
+    // slots nobody reads any more.
+    auto advance = [&]() {
+        a_next += BK;
+        b_next += b_inc;
+        if (++kc_next == nkc) {
+            kc_next = 0;
+            a_next += a_wrap;
+            if (++pos_next == 16) {
+                pos_next = 0;
+                a_next = TI + m0 * C;
+                b_next = Wt;
+            }
+        }
+        lds_next += STAGE_FLOATS * 4;
+        if (++slot_next == NSTAGE) {
+            slot_next = 0;
+            lds_next = smem_base + wave_lds;
+        }
+    };
+
+    // ---- MFMA operands ---------------------------------------------------------------------
+    // A step's reduction range BK is consumed in two halves of KH groups of 8 indices.  Within
+    // a group, lane group lg feeds indices 4*lg .. 4*lg+3, one per MFMA (the order in which
+    // indices are reduced is free as long as A and B agree), so A comes as one b128 read per
+    // group and B as 4 b32 reads, paired so that they merge into ds_read2_b32.
+    constexpr int KH = KS / 2;
+    struct HalfFrag {
+        float4 a[KH][TM];
+        float b[KH][4][TN];
+    };
+    constexpr int NU = KH * (TM + 2 * TN);   // read units per half: KH*TM b128 + KH*2*TN b32 pairs
+    constexpr int NM = KH * 4 * TM * TN;     // MFMAs per half
+
+    // Per-thread LDS offsets within a stage (A in 16-byte units, B in floats).
+    int a_off[KS][TM];
+#pragma unroll
+    for (int k8 = 0; k8 < KS; ++k8)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+            const int row = wm0 + tm * 32 + li;
+            a_off[k8][tm] = row * CH + ((2 * k8 + lg) ^ (row % CH));  // in 16-byte units
+        }
+    const int b_off = A_FLOATS + 4 * lg * BN + wn0 + li;
+
+    // Read unit u of half h of the stage at float offset st into F.
+    auto read_unit = [&](HalfFrag &F, int st, int h, int u) {
+        const int k8l = u / (TM + 2 * TN), v = u % (TM + 2 * TN);
+        const int k8 = h * KH + k8l;
+        if (v < TM) {
+            F.a[k8l][v] = reinterpret_cast<const float4 *>(smem)[st / 4 + a_off[k8][v]];
+        } else {
+            const int tn = (v - TM) / 2, tp = (v - TM) % 2;
+            F.b[k8l][2 * tp][tn] = smem[st + b_off + (k8 * 8 + 2 * tp) * BN + tn * 32];
+            F.b[k8l][2 * tp + 1][tn] = smem[st + b_off + (k8 * 8 + 2 * tp + 1) * BN + tn * 32];
+        }
+    };
+    // MFMA i of a half.
+    auto mfma = [&](floatx16 (&P)[TM][TN], const HalfFrag &F, int i) {
+        const int tn = i % TN, tm = (i / TN) % TM, t = (i / (TN * TM)) % 4, k8l = i / (TN * TM * 4);
+        const float4 a4 = F.a[k8l][tm];
+        const float av = t == 0 ? a4.x : t == 1 ? a4.y : t == 2 ? a4.z : a4.w;
+        P[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, F.b[k8l][t][tn], P[tm][tn], 0, 0, 0);
+    };
+
+    // ---- prologue: fill the ring, wait for step 0, read its first half ----------------------
+#pragma unroll
+    for (int i = 0; i < NSTAGE; ++i) {
+#pragma unroll
+        for (int c = 0; c < LPS; ++c) copy(c);
+        advance();
+    }
+    wait_vmcnt<(NSTAGE - 1) * LPS>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    HalfFrag F1, F2;
+#pragma unroll
+    for (int u = 0; u < NU; ++u) read_unit(F1, 0, 0, u);
+
+    // ---- main loop ----------------------------------------------------------------------------
+    // A wave issues at most one instruction every four cycles and an MFMA occupies the matrix
+    // pipe for 64, so everything that is not an MFMA is dealt out between the MFMAs, a few
+    // instructions after each (sched_barrier pins the order):
+    //   first half  (MFMAs on F1): the LDS reads of the step's second half F2;
+    //   second half (MFMAs on F2): after the first MFMA, wait for the tile of step s+1 and
+    //     barrier (everyone now holds step s entirely in registers, so its ring slot is free);
+    //     then this thread's copies of step s+NSTAGE into that slot, one per MFMA, and the LDS
+    //     reads of F1 of step s+1.
+    int st_cur = 0;  // float offset of the ring slot of the current step
+#pragma unroll
+    for (int pos = 0; pos < 16; ++pos) {
+        floatx16 P[TM][TN];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) P[tm][tn][r] = 0.f;
+
+        for (int kc = 0; kc < nkc; ++kc) {
+            const int st_next = st_cur + STAGE_FLOATS == NSTAGE * STAGE_FLOATS ? 0 : st_cur + STAGE_FLOATS;
+
+#pragma unroll
+            for (int i = 0; i < NM; ++i) {
+                mfma(P, F1, i);
+#pragma unroll
+                for (int u = 0; u < NU; ++u)
+                    if (u * NM / NU == i) read_unit(F2, st_cur, 1, u);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+
+#pragma unroll
+            for (int i = 0; i < NM; ++i) {
+                mfma(P, F2, i);
+                if (i == 0) {
+                    // The tile of step s+1 is complete once at most the copies of steps
+                    // s+2 .. s+NSTAGE-1 are outstanding.
+                    wait_vmcnt<(NSTAGE - 2) * LPS>();
+                    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS reads of step s are done
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                }
+#pragma unroll
+                for (int c = 0; c < LPS; ++c)
+                    if (1 + c * (NM - 1) / LPS == i) copy(c);
+#pragma unroll
+                for (int u = 0; u < NU; ++u)
+                    if (1 + u * (NM - 1) / NU == i) read_unit(F1, st_next, 0, u);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            advance();
+            st_cur = st_next;
+        }
+
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            constexpr unsigned long long plus = kPlus, minus = kMinus;
+            const int bit = 4 * pos + j;
+            if ((plus >> bit) & 1ull) {
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < TN; ++tn) Y[j][tm][tn] += P[tm][tn];
+            } else if ((minus >> bit) & 1ull) {
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < TN; ++tn) Y[j][tm][tn] -= P[tm][tn];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn) asm volatile("" : "+v"(Y[j][tm][tn]));
+    }
+
+    // The surplus copies must have landed before this workgroup's LDS can be handed on.
+    wait_vmcnt<0>();
+
+    store_output<Cfg>(Y, Out, M, K, nW, m0, n0, wm0, wn0, li, lg);
+}
+
+}  // namespace
+}  // namespace swc
