@@ -26,6 +26,13 @@ for _p in (ROOT, PKG):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
+# HBM traffic per launch (bytes), measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
+# what the same counters read for a 128 MiB copy (profiles/*_pmc_traffic.md); None where not measured.
+MEASURED_TRAFFIC = {
+    ("cfg3", "fp32", "conv"): 148.0e6,     # 122.3 MB fetched + 25.69 MB written (algorithmic 129.5 MB)
+    ("cfg3", "fp32", "imtrans"): 131.9e6,  # 29.2 MB fetched + 102.76 MB written (algorithmic 128.45 MB)
+}
+
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, datasheet
 FP32_MFMA_PEAK_TF = 157.3  # MI355X dense fp32 matrix, datasheet
 BF16_MFMA_PEAK_TF = 2500.0
@@ -114,7 +121,19 @@ def main():
     ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg and the parity gate")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU work for cpu_baseline")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="run five 128 MiB device-to-device copies and exit: the known-size kernel that the "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled against")
     args = ap.parse_args()
+    if args.copy_probe:
+        import torch
+        a = torch.ones(32 * 1024 * 1024, device="cuda")
+        b = torch.empty_like(a)
+        for _ in range(5):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_bytes_read": a.numel() * 4, "copy_probe_bytes_written": a.numel() * 4}))
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on one GPU only; --gpus %d is not supported (the forward pass "
                  "shards over the batch with no exchange step, so N GPUs are N independent copies of this run)"
@@ -222,7 +241,7 @@ def main():
             "peak": peak_tf,
             "unit": "TFLOP/s",
             "frac": round(tf_conv / peak_tf, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC.get((name, args.precision, "conv")),
             "algorithmic_flop_per_launch": gemm_flops,
             "algorithmic_bytes_per_launch": conv_bytes,
         },
@@ -233,7 +252,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs_imtrans / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC.get((name, "fp32", "imtrans")),
             "algorithmic_bytes_per_launch": imtrans_bytes,
         },
     }

@@ -90,7 +90,10 @@ __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__rest
                                                              size_t plane)
 {
     using V = typename Vec<VEC>::type;
-    const Idx idx = static_cast<Idx>(blockIdx.x) * 256 + threadIdx.x;
+    // Consecutive logical blocks share input rows (the halo between tile rows, the overlap
+    // between neighbouring tiles); keeping them on one XCD lets its L2 serve the re-reads
+    // instead of every XCD fetching the same rows again.
+    const Idx idx = static_cast<Idx>(xcd_swizzle(blockIdx.x, gridDim.x)) * 256 + threadIdx.x;
     if (idx >= items) return;
     const int CV = C / VEC;
     const int cv = static_cast<int>(idx % CV);
