@@ -96,6 +96,13 @@ CONV_SHAPES = [
     (8, 7, 7, 256, 256),   # config 4a
     (8, 4, 4, 512, 512),   # config 4b
     (1, 2, 2, 1028, 12),
+    # shapes that steer the launcher onto each of its kernels and their ragged edges
+    (2, 3, 5, 64, 100),    # copy-ring kernel, 32-channel steps: rows and columns beyond the last tile
+    (1, 5, 7, 48, 20),     # copy-ring kernel, 16-channel steps (C % 32 != 0), K below one tile
+    (3, 7, 7, 32, 64),     # a single 32-channel step per position
+    (2, 3, 3, 96, 132),    # K = 2 tiles + 4 columns
+    (1, 1, 1, 32, 4),      # one tile row, one column group
+    (5, 9, 11, 160, 72),   # M = 495 (ragged last tile), C = 5 steps
 ]
 
 
