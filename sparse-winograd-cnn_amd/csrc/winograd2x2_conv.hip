@@ -48,7 +48,7 @@ bool async_eligible(const float *TI, const float *Wt, int C, int K)
            static_cast<size_t>(Cfg::BM) * C < (1ull << 29) && static_cast<size_t>(Cfg::BK) * K < (1ull << 29);
 }
 
-template <typename Cfg, int NSTAGE>
+template <typename Cfg, int NSTAGE, bool BF16>
 int launch_async(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nH, int nW,
                  hipStream_t stream)
 {
@@ -56,7 +56,7 @@ int launch_async(const float *TI, const float *Wt, float *Out, size_t M, int C, 
     const size_t tiles_n = (static_cast<size_t>(K) + Cfg::BN - 1) / Cfg::BN;
     if (tiles_m * tiles_n >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
     const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n)), block(Cfg::NT);
-    conv_mfma_async_kernel<Cfg, NSTAGE><<<grid, block, 0, stream>>>(TI, Wt, Out, M, C, K, nH, nW,
+    conv_mfma_async_kernel<Cfg, NSTAGE, BF16><<<grid, block, 0, stream>>>(TI, Wt, Out, M, C, K, nH, nW,
                                                                     static_cast<unsigned>(tiles_n));
     return check_launch();
 }
@@ -73,12 +73,12 @@ int conv_entry(const float *Input, const float *Weight, float *Output, int C, in
     hipStream_t s = static_cast<hipStream_t>(stream);
     using Tile32 = ConvCfg<64, 64, 32, 2, 2>;
     using Tile16 = ConvCfg<64, 64, 16, 2, 2>;
-    if (!BF16) {
-        if (async_eligible<Tile32>(Input, Weight, C, K))
-            return launch_async<Tile32, 2>(Input, Weight, Output, M, C, K, nH, nW, s);
-        if (async_eligible<Tile16>(Input, Weight, C, K))
-            return launch_async<Tile16, 3>(Input, Weight, Output, M, C, K, nH, nW, s);
-    }
+    // Ring depth: the fp32 step is long (16 MFMAs of 64 cycles per wave) and one tile in flight
+    // covers the memory latency; the bf16 step is 8x shorter and needs two.
+    if (async_eligible<Tile32>(Input, Weight, C, K))
+        return launch_async<Tile32, BF16 ? 3 : 2, BF16>(Input, Weight, Output, M, C, K, nH, nW, s);
+    if (!BF16 && async_eligible<Tile16>(Input, Weight, C, K))
+        return launch_async<Tile16, 3, false>(Input, Weight, Output, M, C, K, nH, nW, s);
     return launch_sync<Tile32, BF16>(Input, Weight, Output, M, C, K, nH, nW, s);
 }
 

@@ -2,6 +2,8 @@
 // See winograd2x2_conv.hip for what it replaces in the reference.
 #pragma once
 
+#include <type_traits>
+
 #include "swc_common.h"
 
 namespace swc {
@@ -9,6 +11,20 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// Calls f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N-1>{}) in order: a loop
+// whose index is a compile-time constant in every iteration.
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
 
 // Signs of A^T (x) A^T: bit (4*i + j) set when +-P_i enters Y_j, j = 2*dy + dx.
 // Row i = 4r+s contributes AT[dy][r]*AT[dx][s] with AT = [[1,1,1,0],[0,1,-1,-1]]
@@ -374,7 +390,11 @@ __device__ __forceinline__ void wait_vmcnt()
     asm volatile("" ::: "memory");
 }
 
-template <typename Cfg, int NSTAGE>
+// BF16: the operands are rounded to bf16 (round-to-nearest-even, v_cvt_pk_bf16_f32) after they are read
+// from LDS and multiplied with v_mfma_f32_32x32x16_bf16; accumulation, fold and stores stay fp32.
+// ABL: timing ablations for kernel development (bit 0: no barrier, 1: no copy wait, 2: no copies,
+// 3: no LDS reads); results are wrong with any bit set.  Always 0 in the library.
+template <typename Cfg, int NSTAGE, bool BF16 = false, int ABL = 0>
 __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_mfma_async_kernel(
     const float *__restrict__ TI, const float *__restrict__ Wt, float *__restrict__ Out, size_t M, int C, int K, int nH,
     int nW, unsigned tiles_n)
@@ -386,6 +406,7 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     constexpr int LPS = NA + NB;  // loads per thread per step
     static_assert(NSTAGE >= 2, "a ring needs two slots");
     static_assert(KS % 2 == 0, "the MFMA chain of a step is split in two halves");
+    static_assert(!BF16 || KS == 4, "the bf16 MFMA consumes 16 reduction indices: a half of a 32-index step");
     static_assert((CH & (CH - 1)) == 0, "swizzle needs a power-of-two chunk count");
     static_assert(BM % (64 / CH) == 0 && (BM * CH) % 64 == 0 && (BK * BN / 4) % 64 == 0, "whole wave-loads");
     static_assert((NSTAGE - 2) * LPS < 64, "vmcnt range");
@@ -485,7 +506,8 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
         float b[KH][4][TN];
     };
     constexpr int NU = KH * (TM + 2 * TN);   // read units per half: KH*TM b128 + KH*2*TN b32 pairs
-    constexpr int NM = KH * 4 * TM * TN;     // MFMAs per half
+    // MFMAs per half: fp32 32x32x2 reduces 2 indices each, bf16 32x32x16 all 16 of a half at once.
+    constexpr int NM = BF16 ? TM * TN : KH * 4 * TM * TN;
 
     // Per-thread LDS offsets within a stage (A in 16-byte units, B in floats).
     int a_off[KS][TM];
@@ -510,14 +532,6 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
             F.b[k8l][2 * tp + 1][tn] = smem[st + b_off + (k8 * 8 + 2 * tp + 1) * BN + tn * 32];
         }
     };
-    // MFMA i of a half.
-    auto mfma = [&](floatx16 (&P)[TM][TN], const HalfFrag &F, int i) {
-        const int tn = i % TN, tm = (i / TN) % TM, t = (i / (TN * TM)) % 4, k8l = i / (TN * TM * 4);
-        const float4 a4 = F.a[k8l][tm];
-        const float av = t == 0 ? a4.x : t == 1 ? a4.y : t == 2 ? a4.z : a4.w;
-        P[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, F.b[k8l][t][tn], P[tm][tn], 0, 0, 0);
-    };
-
     // ---- prologue: fill the ring, wait for step 0, read its first half ----------------------
 #pragma unroll
     for (int i = 0; i < NSTAGE; ++i) {
@@ -541,75 +555,112 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     //     barrier (everyone now holds step s entirely in registers, so its ring slot is free);
     //     then this thread's copies of step s+NSTAGE into that slot, one per MFMA, and the LDS
     //     reads of F1 of step s+1.
+    //
+    // The fold of a finished position into Y (up to 4*TM*TN vector adds) is dealt out the same
+    // way over the first step of the next position, which accumulates into the other of two
+    // product buffers and starts its chains from a zero accumulator.
     int st_cur = 0;  // float offset of the ring slot of the current step
-#pragma unroll
-    for (int pos = 0; pos < 16; ++pos) {
-        floatx16 P[TM][TN];
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-            for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) P[tm][tn][r] = 0.f;
+    floatx16 P[2][TM][TN];
+    const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-        for (int kc = 0; kc < nkc; ++kc) {
-            const int st_next = st_cur + STAGE_FLOATS == NSTAGE * STAGE_FLOATS ? 0 : st_cur + STAGE_FLOATS;
-
-#pragma unroll
-            for (int i = 0; i < NM; ++i) {
-                mfma(P, F1, i);
-#pragma unroll
-                for (int u = 0; u < NU; ++u)
-                    if (u * NM / NU == i) read_unit(F2, st_cur, 1, u);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-
-#pragma unroll
-            for (int i = 0; i < NM; ++i) {
-                mfma(P, F2, i);
-                if (i == 0) {
-                    // The tile of step s+1 is complete once at most the copies of steps
-                    // s+2 .. s+NSTAGE-1 are outstanding.
-                    wait_vmcnt<(NSTAGE - 2) * LPS>();
-                    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS reads of step s are done
-                    __builtin_amdgcn_s_barrier();
-                    asm volatile("" ::: "memory");
-                }
-#pragma unroll
-                for (int c = 0; c < LPS; ++c)
-                    if (1 + c * (NM - 1) / LPS == i) copy(c);
-#pragma unroll
-                for (int u = 0; u < NU; ++u)
-                    if (1 + u * (NM - 1) / NU == i) read_unit(F1, st_next, 0, u);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            advance();
-            st_cur = st_next;
+    // Fold unit e of position `pos` (e = j*TM*TN + tm*TN + tn): Y_j +-= P.  The empty asm pins the
+    // update here: Y is not read again until the final stores, so without it the compiler defers
+    // all the adds to the end and keeps the 16 product tiles alive instead of the 4 sums.
+    constexpr int NE = 4 * TM * TN;
+    auto fold_unit = [&](const floatx16 (&Pp)[TM][TN], int pos, int e) {
+        constexpr unsigned long long plus = kPlus, minus = kMinus;
+        const int j = e / (TM * TN), tm = (e / TN) % TM, tn = e % TN;
+        const int bit = 4 * pos + j;
+        if ((plus >> bit) & 1ull) {
+            Y[j][tm][tn] += Pp[tm][tn];
+            asm volatile("" : "+v"(Y[j][tm][tn]));
+        } else if ((minus >> bit) & 1ull) {
+            Y[j][tm][tn] -= Pp[tm][tn];
+            asm volatile("" : "+v"(Y[j][tm][tn]));
         }
+    };
 
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            constexpr unsigned long long plus = kPlus, minus = kMinus;
-            const int bit = 4 * pos + j;
-            if ((plus >> bit) & 1ull) {
-#pragma unroll
-                for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-                    for (int tn = 0; tn < TN; ++tn) Y[j][tm][tn] += P[tm][tn];
-            } else if ((minus >> bit) & 1ull) {
-#pragma unroll
-                for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-                    for (int tn = 0; tn < TN; ++tn) Y[j][tm][tn] -= P[tm][tn];
+    // One step.  first: the chains start from zero and the fold of position fold_pos (held in
+    // Pprev) rides along; otherwise fold_pos is ignored.
+    auto step = [&](floatx16 (&Pc)[TM][TN], const floatx16 (&Pprev)[TM][TN], auto first_tag, auto fold_tag) {
+        constexpr bool first = decltype(first_tag)::value;
+        constexpr int fold_pos = decltype(fold_tag)::value;
+        const int st_next = st_cur + STAGE_FLOATS == NSTAGE * STAGE_FLOATS ? 0 : st_cur + STAGE_FLOATS;
+        auto mfma_slot = [&](const HalfFrag &F, int i, bool from_zero) {
+            if constexpr (BF16) {
+                // Lane group lg holds reduction indices {8*k8l + 4*lg + t}: 8 per half, the same
+                // set on the A and the B side, which is all the MFMA needs.
+                const int tn = i % TN, tm = i / TN;
+                const float4 a0 = F.a[0][tm], a1 = F.a[1][tm];
+                auto pk = [](float x, float y) { return __builtin_convertvector(floatx2{x, y}, bf16x2); };
+                const bf16x2 p0 = pk(a0.x, a0.y), p1 = pk(a0.z, a0.w), p2 = pk(a1.x, a1.y), p3 = pk(a1.z, a1.w);
+                const bf16x2 q0 = pk(F.b[0][0][tn], F.b[0][1][tn]), q1 = pk(F.b[0][2][tn], F.b[0][3][tn]);
+                const bf16x2 q2 = pk(F.b[1][0][tn], F.b[1][1][tn]), q3 = pk(F.b[1][2][tn], F.b[1][3][tn]);
+                const bf16x8 av = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+                const bf16x8 bv = {q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
+                Pc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, from_zero ? zero16 : Pc[tm][tn], 0, 0, 0);
+            } else {
+                const int tn = i % TN, tm = (i / TN) % TM, t = (i / (TN * TM)) % 4, k8l = i / (TN * TM * 4);
+                const float4 a4 = F.a[k8l][tm];
+                const float av = t == 0 ? a4.x : t == 1 ? a4.y : t == 2 ? a4.z : a4.w;
+                Pc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, F.b[k8l][t][tn], from_zero ? zero16 : Pc[tm][tn], 0, 0, 0);
             }
+        };
+        // Slots (MFMA indices of the second half) after which the copies and LDS reads go; all
+        // behind the barrier that follows MFMA 0.
+        auto copy_slot = [](int c) { return NM > 1 ? 1 + c * (NM - 1) / LPS : 0; };
+        auto read_slot = [](int u) { return NM > 1 ? 1 + u * (NM - 1) / NU : 0; };
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            mfma_slot(F1, i, first && i < TM * TN);
+#pragma unroll
+            for (int u = 0; u < NU; ++u)
+                if (u * NM / NU == i && !(ABL & 8)) read_unit(F2, st_cur, 1, u);
+            if (first && fold_pos >= 0) {
+#pragma unroll
+                for (int e = 0; e < NE; ++e)
+                    if (e * (2 * NM) / NE == i) fold_unit(Pprev, fold_pos, e);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int i = 0; i < NM; ++i) {
+            mfma_slot(F2, i, false);
+            if (i == 0) {
+                // The tile of the next step is complete once at most the copies of the NSTAGE-2
+                // steps after it are outstanding.
+                if (!(ABL & 2)) wait_vmcnt<(NSTAGE - 2) * LPS>();
+                __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS reads of this step are done
+                if (!(ABL & 1)) __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            }
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm)
+            for (int c = 0; c < LPS; ++c)
+                if (copy_slot(c) == i && !(ABL & 4)) copy(c);
 #pragma unroll
-                for (int tn = 0; tn < TN; ++tn) asm volatile("" : "+v"(Y[j][tm][tn]));
-    }
+            for (int u = 0; u < NU; ++u)
+                if (read_slot(u) == i && !(ABL & 8)) read_unit(F1, st_next, 0, u);
+            if (first && fold_pos >= 0) {
+#pragma unroll
+                for (int e = 0; e < NE; ++e)
+                    if (e * (2 * NM) / NE == NM + i) fold_unit(Pprev, fold_pos, e);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        advance();
+        st_cur = st_next;
+    };
+
+    // The position loop is unrolled at compile time so that the signs of the output transform
+    // are constants (a run-time loop over position pairs with branched folds measured 6 % slower).
+    static_for<16>([&](auto pos_tag) {
+        constexpr int pos = decltype(pos_tag)::value;
+        step(P[pos & 1], P[(pos & 1) ^ 1], std::true_type{}, std::integral_constant<int, pos - 1>{});
+        for (int kc = 1; kc < nkc; ++kc)
+            step(P[pos & 1], P[(pos & 1) ^ 1], std::false_type{}, std::integral_constant<int, -1>{});
+    });
+#pragma unroll
+    for (int e = 0; e < NE; ++e) fold_unit(P[1], 15, e);
 
     // The surplus copies must have landed before this workgroup's LDS can be handed on.
     wait_vmcnt<0>();
