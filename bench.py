@@ -112,12 +112,56 @@ def cpu_baseline(name, x, w, budget_s):
     }, ti, y
 
 
+def bench_resnet(args, torch, dev):
+    """BASELINE config 5: full ResNet-18-var forward, all 16 3x3 convs through the ops, random-init weights
+    magnitude-pruned per layer (30/20/10/10 % density by stage), input ~N(0,1) [N,224,224,3]."""
+    import numpy as np
+
+    import resnet18_var
+    from winograd_weights import gen_prune_mask
+
+    rng = np.random.default_rng(500)
+    density = {"2": 0.3, "3": 0.2, "4": 0.1, "5": 0.1}
+    model = resnet18_var.ResNet18Var(precision=args.precision)
+    for lname, conv in zip(resnet18_var.winograd_layer_names(), model.winograd_convs()):
+        w = conv.W.data.numpy().copy()
+        conv.mask = torch.from_numpy(gen_prune_mask(w, density[lname[len("Winograd_W")]]))
+    model = model.to(dev)
+    N = args.batch
+    image = torch.from_numpy(rng.standard_normal((N, 224, 224, 3)).astype(np.float32)).to(dev)
+    # 18*N*H*W*C*K over the 16 Winograd layers at the sizes the model runs them (56, 28, 14, 14)
+    sizes = {"2": 56, "3": 28, "4": 14, "5": 14}
+    flops = sum(18.0 * N * sizes[n[len("Winograd_W")]] ** 2 * c.in_channel * c.out_channel
+                for n, c in zip(resnet18_var.winograd_layer_names(), model.winograd_convs()))
+    for _ in range(max(args.warmup // 4, 2)):
+        logits = model(image)
+    torch.cuda.synchronize()
+    steps = max(args.steps // 10, 5)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        logits = model(image)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    print(json.dumps({
+        "metric": "ResNet-18-var Winograd-ReLU forward (config 5), effective conv GFLOP/s of its 16 3x3 layers",
+        "value": round(flops / (ms * 1e-3) / 1e9, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": steps,
+        "warmup": max(args.warmup // 4, 2), "ms_per_step": round(ms, 3), "images_per_s": round(N / (ms * 1e-3), 1),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if args.precision == "fp32" else "bf16 operands, f32 accumulate", "data": "synthetic",
+        "config": {"workload": "cfg5: ResNet-18-var forward, N=%d, 224x224x3, whole model time incl. stock "
+                               "PyTorch conv1/1x1/BN/pool/FC" % N, "gemm_precision": args.precision},
+        "logits_finite": bool(torch.isfinite(logits).all()),
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg5"],
+                    help="cfg1-cfg4b: one layer; cfg5: the whole ResNet-18-var forward (16 Winograd layers), N=128")
+    ap.add_argument("--batch", type=int, default=128, help="batch size of the cfg5 forward")
     ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg and the parity gate")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU work for cpu_baseline")
@@ -155,6 +199,8 @@ def main():
           getattr(prop, "clock_rate", 0) / 1e3, prop.total_memory / 2 ** 30), file=sys.stderr)
 
     name = args.workload
+    if name == "cfg5":
+        return bench_resnet(args, torch, dev)
     B, H, W, C, K, density, kind = WORKLOADS[name]
     nH, nW = (H + 1) // 2, (W + 1) // 2
     M = B * nH * nW

@@ -1,0 +1,116 @@
+"""Forward pass of the reference's ResNet-18 variant with its sixteen 3x3 convolutions routed
+through the Winograd-ReLU ops (inference only).
+
+Topology after ``Model._build_graph`` in ResNet-18-var/imagenet-resnet-transWino-prune.py:109-220:
+conv1 7x7/2 (no BN, :113) -> pool 3/2 (:115); four stages of two residual units; every unit is
+``BN -> WinogradImTrans(relu) -> WinogradConv -> BN -> WinogradImTrans(relu) -> WinogradConv -> BN``
+(:117-123 ...), the first unit of a stage adds a 1x1 shortcut conv + BN (:126-129, :152-155, ...);
+3/2 max-pools close stages 2 and 3 (:141,:166) but not stage 4 (pool4 is commented out, :191), so
+stage 5 also runs at 14x14; ReLU, global average pool, (dropout: identity at inference), FC 1000
+(:213-219).  Padding of the strided conv and the pools is TensorFlow's SAME (the extra pixel goes
+after, not before).
+
+Everything except the two Winograd ops is stock PyTorch.  Activations are kept NHWC in memory
+(channels_last), so handing them to the ops and back costs no copies.
+"""
+import os
+import sys
+
+import torch
+import torch.nn.functional as F
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+from winograd_conv import WinogradConv  # noqa: E402
+from winograd_imtrans import WinogradImTrans  # noqa: E402
+
+# (unit name, C_in of the first conv, C_out, has 1x1 shortcut conv, max-pool after the unit)
+UNITS = (
+    ("2a", 64, 64, True, False), ("2b", 64, 64, False, True),
+    ("3a", 64, 128, True, False), ("3b", 128, 128, False, True),
+    ("4a", 128, 256, True, False), ("4b", 256, 256, False, False),
+    ("5a", 256, 512, True, False), ("5b", 512, 512, False, False),
+)
+
+
+def winograd_layer_names():
+    """The 16 weight names of the reference graph, in order (Winograd_W2a_2a ... Winograd_W5b_2b)."""
+    return ["Winograd_W%s_2%s" % (u[0], ab) for u in UNITS for ab in "ab"]
+
+
+def _same_pad(x, k, stride):
+    """TensorFlow SAME padding for an NCHW tensor: total = max((ceil(n/s)-1)*s + k - n, 0), smaller half first."""
+    pads = []
+    for n in (x.shape[3], x.shape[2]):  # F.pad wants W first
+        total = max((-(-n // stride) - 1) * stride + k - n, 0)
+        pads += [total // 2, total - total // 2]
+    return pads
+
+
+def _to_nhwc(x):   # NCHW tensor in channels_last memory -> contiguous [B,H,W,C] view
+    return x.permute(0, 2, 3, 1).contiguous()
+
+
+def _to_nchw(y):   # contiguous [B,H,W,C] -> NCHW tensor in channels_last memory (a view)
+    return y.permute(0, 3, 1, 2)
+
+
+class WinogradUnit(torch.nn.Module):
+    def __init__(self, name, c_in, c_out, shortcut, pool, masks, precision):
+        super().__init__()
+        self.name, self.pool = name, pool
+        self.bn2a = torch.nn.BatchNorm2d(c_in)
+        self.conv2a = WinogradConv(c_in, c_out, mask=masks.get("Winograd_W%s_2a/W" % name), precision=precision)
+        self.bn2b = torch.nn.BatchNorm2d(c_out)
+        self.conv2b = WinogradConv(c_out, c_out, mask=masks.get("Winograd_W%s_2b/W" % name), precision=precision)
+        self.bn2c = torch.nn.BatchNorm2d(c_out)
+        self.shortcut = shortcut
+        if shortcut:
+            self.bn_pre = torch.nn.BatchNorm2d(c_in) if name == "2a" else None  # BNReLU('res2a_1_relu') only in 2a
+            self.conv1 = torch.nn.Conv2d(c_in, c_out, 1, bias=False)
+            self.bn1 = torch.nn.BatchNorm2d(c_out)
+
+    def branch(self, x):
+        h = _to_nchw(self.conv2a(WinogradImTrans(_to_nhwc(self.bn2a(x)), torch.relu)))
+        h = _to_nchw(self.conv2b(WinogradImTrans(_to_nhwc(self.bn2b(h)), torch.relu)))
+        return self.bn2c(h)
+
+    def forward(self, x):
+        bra = self.branch(x)
+        if self.shortcut:
+            s = torch.relu(self.bn_pre(x)) if self.bn_pre is not None else torch.relu(x)
+            x = self.bn1(self.conv1(s))
+        else:
+            x = torch.relu(x)
+        x = x + bra
+        if self.pool:
+            x = F.max_pool2d(F.pad(x, _same_pad(x, 3, 2), value=float("-inf")), 3, 2)
+        return x
+
+
+class ResNet18Var(torch.nn.Module):
+    """``masks``: optional dict of 0/1 arrays keyed like the reference's pruning masks
+    ('Winograd_W2a_2a/W', ...; prune_script.py:68-78).  ``precision``: 'fp32' or 'bf16' GEMM operands."""
+
+    def __init__(self, masks=None, precision="fp32", num_classes=1000):
+        super().__init__()
+        masks = masks or {}
+        self.conv1 = torch.nn.Conv2d(3, 64, 7, stride=2, bias=False)
+        self.units = torch.nn.ModuleList(
+            [WinogradUnit(n, ci, co, sc, pool, masks, precision) for n, ci, co, sc, pool in UNITS])
+        self.linear = torch.nn.Linear(512, num_classes)
+        self.eval()
+
+    def winograd_convs(self):
+        return [c for u in self.units for c in (u.conv2a, u.conv2b)]
+
+    @torch.no_grad()
+    def forward(self, image):
+        """image: [B,H,W,3] float32 NHWC (already normalised) -> logits [B,num_classes]."""
+        x = image.permute(0, 3, 1, 2)  # NCHW view over NHWC memory = channels_last
+        x = self.conv1(F.pad(x, _same_pad(x, 7, 2)))
+        x = F.max_pool2d(F.pad(x, _same_pad(x, 3, 2), value=float("-inf")), 3, 2)
+        x = x.contiguous(memory_format=torch.channels_last)
+        for unit in self.units:
+            x = unit(x)
+        x = torch.relu(x).mean(dim=(2, 3))
+        return self.linear(x)
