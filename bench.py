@@ -165,6 +165,9 @@ def main():
     ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg and the parity gate")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU work for cpu_baseline")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time the two gradient ops (conv grad: dP transform + two rocBLAS batched GEMMs; "
+                         "imTrans grad with the ReLU mask) and add a `backward` object to the line")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run five 128 MiB device-to-device copies and exit: the known-size kernel that the "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled against")
@@ -305,6 +308,36 @@ def main():
             "algorithmic_bytes_per_launch": imtrans_bytes,
         },
     }
+
+    if args.backward:
+        dy = torch.randn(B, 2 * nH, 2 * nW, K, device=dev)
+        dti, dw = torch.empty_like(ti), torch.empty_like(w)
+        tmp = torch.empty(16 * M * K, device=dev)
+        dx = torch.empty(B, 2 * nH, 2 * nW, C, device=dev)
+        ptr = lambda t: t.data_ptr()  # noqa: E731
+
+        def f_conv_grad():
+            if L.swc_winograd2x2_conv_grad(tip, wp, ptr(dy), ptr(dti), ptr(dw), ptr(tmp), None, C, B, 2 * nH, 2 * nW, K,
+                                           1, 1, stream) != 0:
+                raise RuntimeError("swc_winograd2x2_conv_grad failed")
+
+        def f_imtrans_grad():
+            if L.swc_winograd2x2_imtrans_grad(ptr(dti), tip, ptr(dx), C, B, 2 * nH, 2 * nW, 1, 1, stream) != 0:
+                raise RuntimeError("swc_winograd2x2_imtrans_grad failed")
+
+        for _ in range(3):
+            f_conv_grad()
+            f_imtrans_grad()
+        iters = max(args.steps // 4, 10)
+        ms_cg = time_loop(f_conv_grad, iters, torch)
+        ms_ig = time_loop(f_imtrans_grad, iters, torch)
+        out["backward"] = {
+            "ms_conv_grad": round(ms_cg, 5),
+            "conv_grad_TFLOPs": round(2 * gemm_flops / (ms_cg * 1e-3) / 1e12, 2),  # two GEMMs of 32*M*C*K each
+            "ms_imtrans_grad": round(ms_ig, 5),
+            # reads dT and the mask source (2 * 64*M*C bytes), writes dX
+            "imtrans_grad_GBps": round((128.0 * M * C + 4.0 * B * 4 * nH * nW * C) / (ms_ig * 1e-3) / 1e9, 1),
+        }
 
     if not args.no_cpu:
         cpu, ti_ref, y32_ref = cpu_baseline(name, x_np, w_np, args.cpu_budget)

@@ -131,6 +131,44 @@ SWC_API int swc_winograd2x2_conv_op_compute(const float *input, int in_rank, con
                                     float *output, int out_rank, const int64_t *out_dims,
                                     int precision, swc_stream_t stream);
 
+/* ---------------------------------------------------------------------------
+ * Backward ops.
+ * ------------------------------------------------------------------------- */
+
+/*
+ * Gradient of swc_winograd2x2_conv with respect to both inputs.
+ *   TInput [16,B,nH,nW,C], Weight [16,C,K], Output_grad [B,H,W,K] with H = 2nH, W = 2nW
+ *   -> TInput_grad [16,B,nH,nW,C], Weight_grad [16,C,K]
+ * Replaces  void Winograd2x2ConvGradComputeLauncher(const float *TInput, const float *Weight,
+ *           const float *Output_grad, float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,
+ *           long long *tmp_ptr_buffer, int C, int B, int H, int W, int K, int pad_h, int pad_w)
+ *   declared winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_grad_op.cc:32,
+ *   defined  winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_grad_cuda.cu.cc:77-124.
+ * tmp_data_buffer must hold 16*B*nH*nW*K floats (the caller's temporary, as at
+ * winograd2x2_conv_grad_op.cc:69-71); tmp_ptr_buffer is ignored.  The two batched GEMMs run in
+ * rocBLAS; the first call on a host thread creates that thread's rocBLAS handle, which is the one
+ * piece of state (and device memory) this library ever owns.
+ */
+SWC_API int swc_winograd2x2_conv_grad(const float *TInput, const float *Weight, const float *Output_grad,
+                                      float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,
+                                      long long *tmp_ptr_buffer, int C, int B, int H, int W, int K,
+                                      int pad_h, int pad_w, swc_stream_t stream);
+
+/*
+ * Gradient of swc_winograd2x2_imtrans: TransIm_grad [16,B,nH,nW,C] -> Input_grad [B,H,W,C].
+ * Replaces  void Winograd2x2ImTransGradComputeLauncher(const float *Output_grad, float *Input_grad,
+ *           int C, int B, int H, int W, int pad_h, int pad_w)
+ *   declared winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans_grad_op.cc:29,
+ *   defined  winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans_grad_cuda.cu.cc:118-129.
+ * relu_mask_source, if not NULL, is the forward op's output computed with relu != 0: the gradient
+ * is then taken through the fused ReLU (entries where it is <= 0 contribute nothing).  Unlike the
+ * reference (:124), TransIm_grad is not overwritten.  H need not be even here (the reference's op
+ * wrapper always passes H = 2nH, winograd2x2_imTrans_grad_op.cc:44-45).
+ */
+SWC_API int swc_winograd2x2_imtrans_grad(const float *TransIm_grad, const float *relu_mask_source,
+                                         float *Input_grad, int C, int B, int H, int W,
+                                         int pad_h, int pad_w, swc_stream_t stream);
+
 #ifdef __cplusplus
 } /* extern "C" */
 
@@ -146,6 +184,13 @@ SWC_API void Winograd2x2ImTransComputeLauncher(const float *Input, float *TransI
 SWC_API void Winograd2x2ConvComputeLauncher(const float *Input, const float *Weight, float *Output,
                                     float *tmp_data_buffer, const long long *tmp_ptr_buffer,
                                     int C, int B, int nH, int nW, int K, int pad_h, int pad_w);
+/* Likewise for the gradient ops (winograd2x2_conv_grad_op.cc:32,77; winograd2x2_imTrans_grad_op.cc:29,54). */
+SWC_API void Winograd2x2ConvGradComputeLauncher(const float *TInput, const float *Weight, const float *Output_grad,
+                                        float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,
+                                        long long *tmp_ptr_buffer, int C, int B, int H, int W, int K,
+                                        int pad_h, int pad_w);
+SWC_API void Winograd2x2ImTransGradComputeLauncher(const float *Output_grad, float *Input_grad, int C, int B,
+                                           int H, int W, int pad_h, int pad_w);
 #endif
 
 #endif /* WINOGRAD2X2_H_ */

@@ -133,3 +133,55 @@ def gen_prune_mask(mat, density):
     mask[drop] = 0
     np.copyto(mat, flat.reshape(mat.shape))
     return mask.reshape(mat.shape)
+
+
+def _bind_grad():
+    L = lib()
+    if not hasattr(L, "_grad_bound"):
+        L.oracle_output_transform_grad_f32.argtypes = [_F, _F] + [ctypes.c_int] * 4
+        L.oracle_conv_grad_f32.argtypes = [_F, _F, _F, _F, _F, _F] + [ctypes.c_int] * 5
+        L.oracle_imtrans_grad_f32.argtypes = [_F, _F, _F] + [ctypes.c_int] * 4
+        for f in (L.oracle_output_transform_grad_f32, L.oracle_conv_grad_f32, L.oracle_imtrans_grad_f32):
+            f.restype = None
+        L._grad_bound = True
+    return L
+
+
+def output_transform_grad(dy):
+    """dy [B,2nH,2nW,K] -> dP [16,B*nH*nW,K] (A dY A^T per tile)."""
+    dy, dyp = _f32(dy)
+    B, H, W, K = dy.shape
+    nH, nW = H // 2, W // 2
+    out = np.empty((16, B * nH * nW, K), dtype=np.float32)
+    _bind_grad().oracle_output_transform_grad_f32(dyp, out.ctypes.data_as(_F), B, nH, nW, K)
+    return out
+
+
+def conv_grad(ti, w, dy):
+    """Winograd2x2ConvGrad: (ti [16,B,nH,nW,C], w [16,C,K], dy [B,2nH,2nW,K]) -> (dti, dw)."""
+    ti, tp = _f32(ti)
+    w, wp = _f32(w)
+    dy, dyp = _f32(dy)
+    _, B, nH, nW, C = ti.shape
+    K = int(w.shape[2])
+    assert dy.shape == (B, 2 * nH, 2 * nW, K) and w.shape == (16, C, K)
+    dti = np.empty_like(ti)
+    dw = np.empty_like(w)
+    tmp = np.empty(16 * B * nH * nW * K, dtype=np.float32)
+    _bind_grad().oracle_conv_grad_f32(tp, wp, dyp, dti.ctypes.data_as(_F), dw.ctypes.data_as(_F),
+                                     tmp.ctypes.data_as(_F), C, B, nH, nW, K)
+    return dti, dw
+
+
+def imtrans_grad(dt, H, W, mask_src=None):
+    """Winograd2x2ImTransGrad: dt [16,B,nH,nW,C] -> dx [B,H,W,C]; mask_src (post-ReLU TI) applies the ReLU backward."""
+    dt, dtp = _f32(dt)
+    _, B, nH, nW, C = dt.shape
+    assert nH == (H + 1) // 2 and nW == (W + 1) // 2
+    mp = None
+    if mask_src is not None:
+        mask_src, mp = _f32(mask_src)
+        assert mask_src.shape == dt.shape
+    out = np.empty((B, H, W, C), dtype=np.float32)
+    _bind_grad().oracle_imtrans_grad_f32(dtp, mp, out.ctypes.data_as(_F), B, H, W, C)
+    return out

@@ -243,3 +243,130 @@ ORACLE_API void oracle_kernel_transform_f32(const float *g, float *U, int C, int
         for (int i = 0; i < 16; ++i) U[(size_t)i * ck + e] = u[i];
     }
 }
+
+/* ---------------------------------------------------------------------------------------
+ * Backward ops (CVG = winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_grad_cuda.cu.cc,
+ * ITG = winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans_grad_cuda.cu.cc).
+ * Pinned in tests/test_oracle_grad.py by the adjoint identities <f(x), g> == <x, f^T(g)>,
+ * exact on integer inputs, against the forward functions above (which are pinned on their
+ * own), and by float64 matrix forms.
+ * ------------------------------------------------------------------------------------- */
+
+/*
+ * Gradient of the output transform: dP = A dY A^T per tile, [B,2nH,2nW,K] -> [16,B,nH,nW,K].
+ * The 16 expressions of Grad_inverse_transform, CVG:22-43; store order CVG:46-64.
+ */
+ORACLE_API void oracle_output_transform_grad_f32(const float *dY, float *dP, int B, int nH, int nW, int K)
+{
+    const size_t plane = (size_t)B * nH * nW * K;
+    const int H = 2 * nH, W = 2 * nW;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int b = 0; b < B; ++b)
+        for (int th = 0; th < nH; ++th)
+            for (int tw = 0; tw < nW; ++tw) {
+                const float *g0 = dY + (((size_t)b * H + 2 * th) * W + 2 * tw) * K;
+                const float *g1 = g0 + K, *g2 = g0 + (size_t)W * K, *g3 = g2 + K;
+                float *dst = dP + (((size_t)b * nH + th) * nW + tw) * K;
+                for (int k = 0; k < K; ++k) {
+                    const float a = g0[k], bb = g1[k], c = g2[k], d = g3[k];
+                    float p[16];
+                    p[0] = a;          p[1] = a + bb;          p[2] = a - bb;          p[3] = -bb;
+                    p[4] = a + c;      p[5] = a + bb + c + d;  p[6] = a - bb + c - d;  p[7] = -bb - d;
+                    p[8] = a - c;      p[9] = a + bb - c - d;  p[10] = a - bb - c + d; p[11] = d - bb;
+                    p[12] = -c;        p[13] = -c - d;         p[14] = d - c;          p[15] = d;
+                    for (int i = 0; i < 16; ++i) dst[(size_t)i * plane + k] = p[i];
+                }
+            }
+}
+
+/*
+ * Winograd2x2ConvGrad (launcher CVG:77-124): dP as above, then per position
+ *   dTI[i] (M x C) = dP[i] (M x K) . W[i]^T      (cublasSgemmBatched T,N  CVG:103-108)
+ *   dW[i]  (C x K) = TI[i]^T (C x M) . dP[i]     (cublasSgemmBatched N,T  CVG:115-120)
+ * accumulated in float64.  tmp holds 16*M*K floats (conv_grad_op.cc:68-70).
+ */
+ORACLE_API void oracle_conv_grad_f32(const float *TI, const float *Wt, const float *dY, float *dTI, float *dW,
+                                     float *tmp, int C, int B, int nH, int nW, int K)
+{
+    const long M = (long)B * nH * nW;
+    oracle_output_transform_grad_f32(dY, tmp, B, nH, nW, K);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int i = 0; i < 16; ++i)
+        for (long m = 0; m < M; ++m) {
+            const float *dp = tmp + ((size_t)i * M + m) * K;
+            float *o = dTI + ((size_t)i * M + m) * C;
+            for (int c = 0; c < C; ++c) {
+                const float *w = Wt + ((size_t)i * C + c) * K;
+                double acc = 0.0;
+                for (int k = 0; k < K; ++k) acc += (double)dp[k] * (double)w[k];
+                o[c] = (float)acc;
+            }
+        }
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int i = 0; i < 16; ++i)
+        for (int c = 0; c < C; ++c) {
+            double acc[K];
+            for (int k = 0; k < K; ++k) acc[k] = 0.0;
+            for (long m = 0; m < M; ++m) {
+                const double a = (double)TI[((size_t)i * M + m) * C + c];
+                const float *dp = tmp + ((size_t)i * M + m) * K;
+                for (int k = 0; k < K; ++k) acc[k] += a * (double)dp[k];
+            }
+            for (int k = 0; k < K; ++k) dW[((size_t)i * C + c) * K + k] = (float)acc[k];
+        }
+}
+
+/*
+ * Winograd2x2ImTransGrad: dX = sum over tiles of (B dT B^T) scattered back onto the 4x4 patch the
+ * tile was gathered from (pixels outside the image drop out).  dT [16,B,nH,nW,C] -> dX [B,H,W,C].
+ * The per-tile matrix follows OutputGradTransform ITG:39-62; the placement follows the gather of
+ * Winograd2x2ImTransGradCompute ITG:98-114 (tile (h_col,w_col), patch offset (y+1-2h_col, x+1-2w_col)).
+ * If `mask_src` is not NULL, dT is first multiplied by (mask_src > 0): the backward of the fused
+ * Winograd-domain ReLU, mask_src being the forward op's (post-ReLU) output.
+ * Unlike the reference, the incoming gradient is left untouched (ITG:124 overwrites it).
+ */
+ORACLE_API void oracle_imtrans_grad_f32(const float *dT, const float *mask_src, float *dX, int B, int H, int W, int C)
+{
+    const int nH = (H + 1) / 2, nW = (W + 1) / 2;
+    const size_t plane = (size_t)B * nH * nW * C;
+    memset(dX, 0, sizeof(float) * (size_t)B * H * W * C);
+#pragma omp parallel for schedule(static)
+    for (int b = 0; b < B; ++b) {
+        double *acc = (double *)__builtin_malloc(sizeof(double) * (size_t)H * W * C);
+        for (size_t e = 0; e < (size_t)H * W * C; ++e) acc[e] = 0.0;
+        for (int th = 0; th < nH; ++th)
+            for (int tw = 0; tw < nW; ++tw)
+                for (int c = 0; c < C; ++c) {
+                    const size_t off = (((size_t)b * nH + th) * nW + tw) * C + c;
+                    double t[16], d[16];
+                    for (int i = 0; i < 16; ++i) {
+                        t[i] = (double)dT[(size_t)i * plane + off];
+                        if (mask_src && !(mask_src[(size_t)i * plane + off] > 0.0f)) t[i] = 0.0;
+                    }
+                    d[0] = t[0];
+                    d[1] = t[1] - t[2] + t[3];
+                    d[2] = t[1] - t[0] + t[2];
+                    d[3] = -t[3];
+                    d[4] = t[4] - t[8] + t[12];
+                    d[5] = t[5] - t[6] + t[7] - t[9] + t[10] - t[11] + t[13] - t[14] + t[15];
+                    d[6] = t[5] - t[4] + t[6] + t[8] - t[9] - t[10] - t[12] + t[13] + t[14];
+                    d[7] = t[11] - t[7] - t[15];
+                    d[8] = t[4] - t[0] + t[8];
+                    d[9] = t[2] - t[1] - t[3] + t[5] - t[6] + t[7] + t[9] - t[10] + t[11];
+                    d[10] = t[0] - t[1] - t[2] - t[4] + t[5] + t[6] - t[8] + t[9] + t[10];
+                    d[11] = t[3] - t[7] - t[11];
+                    d[12] = -t[12];
+                    d[13] = t[14] - t[13] - t[15];
+                    d[14] = t[12] - t[13] - t[14];
+                    d[15] = t[15];
+                    for (int r = 0; r < 4; ++r)
+                        for (int s = 0; s < 4; ++s) {
+                            const int y = 2 * th - 1 + r, x = 2 * tw - 1 + s;
+                            if (y > -1 && y < H && x > -1 && x < W) acc[((size_t)y * W + x) * C + c] += d[4 * r + s];
+                        }
+                }
+        float *o = dX + (size_t)b * H * W * C;
+        for (size_t e = 0; e < (size_t)H * W * C; ++e) o[e] = (float)acc[e];
+        __builtin_free(acc);
+    }
+}

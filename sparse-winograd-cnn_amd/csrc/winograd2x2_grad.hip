@@ -1,0 +1,243 @@
+// Backward of the two Winograd ops for gfx950.
+//
+// Stand in for Winograd2x2ConvGradComputeLauncher
+// (winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_grad_cuda.cu.cc:77-124) and
+// Winograd2x2ImTransGradComputeLauncher
+// (winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans_grad_cuda.cu.cc:118-129).
+//
+// Conv grad keeps the reference's structure: dP = A dY A^T into the caller's 16*M*K temporary,
+// then two plain batched GEMMs (dTI = dP . W^T, dW = TI^T . dP), here rocBLAS strided-batched
+// SGEMM where the reference calls cublasSgemmBatched.  ImTrans grad is one gather kernel: every
+// input pixel collects, from the up to 2x2 tiles that cover it, its entry of B dT B^T, recomputed
+// from the (at most 9) transform-domain gradients it depends on; the incoming gradient is not
+// modified (the reference transforms it in place first, :124).
+
+#include <cstdio>
+
+#include <rocblas/rocblas.h>
+
+#include "swc_common.h"
+
+namespace swc {
+namespace {
+
+// ---- dP = A dY A^T (Grad_inverse_transform, winograd2x2_conv_grad_cuda.cu.cc:12-66) -------------
+template <int VEC>
+struct GVec;
+template <>
+struct GVec<1> {
+    using type = float;
+};
+template <>
+struct GVec<4> {
+    using type = float4;
+};
+__device__ __forceinline__ float neg(float a) { return -a; }
+__device__ __forceinline__ float4 neg(float4 a) { return make_float4(-a.x, -a.y, -a.z, -a.w); }
+__device__ __forceinline__ float add(float a, float b) { return a + b; }
+__device__ __forceinline__ float sub(float a, float b) { return a - b; }
+__device__ __forceinline__ float4 add(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+__device__ __forceinline__ float4 sub(float4 a, float4 b) { return make_float4(a.x - b.x, a.y - b.y, a.z - b.z, a.w - b.w); }
+
+// One lane per (tile, VEC output channels), numbered along the flattened [M, K/VEC] plane so that
+// each of the 16 stores of a wavefront is contiguous in its plane.
+template <int VEC>
+__global__ __launch_bounds__(256) void output_transform_grad_kernel(const float *__restrict__ dY, float *__restrict__ dP,
+                                                                    int nW, int K, unsigned items, size_t plane)
+{
+    using V = typename GVec<VEC>::type;
+    const unsigned idx = xcd_swizzle(blockIdx.x, gridDim.x) * 256 + threadIdx.x;
+    if (idx >= items) return;
+    const unsigned KV = K / VEC;
+    const unsigned kv = idx % KV, m = idx / KV;
+    const unsigned tw = m % nW, bt = m / nW;  // bt = b*nH + th
+    const size_t oW = 2 * static_cast<size_t>(nW);
+    const float *g = dY + ((static_cast<size_t>(bt) * 2 * oW + 2 * tw) * K + static_cast<size_t>(kv) * VEC);
+    const V a = *reinterpret_cast<const V *>(g), b = *reinterpret_cast<const V *>(g + K);
+    const V c = *reinterpret_cast<const V *>(g + oW * K), d = *reinterpret_cast<const V *>(g + oW * K + K);
+    V p[16];
+    // the expressions of winograd2x2_conv_grad_cuda.cu.cc:28-43, left to right
+    p[0] = a;                           p[1] = add(a, b);                   p[2] = sub(a, b);                   p[3] = neg(b);
+    p[4] = add(a, c);                   p[5] = add(add(add(a, b), c), d);   p[6] = sub(add(sub(a, b), c), d);   p[7] = sub(neg(b), d);
+    p[8] = sub(a, c);                   p[9] = sub(sub(add(a, b), c), d);   p[10] = add(sub(sub(a, b), c), d);  p[11] = sub(d, b);
+    p[12] = neg(c);                     p[13] = sub(neg(c), d);             p[14] = sub(d, c);                  p[15] = d;
+    float *dst = dP + static_cast<size_t>(idx) * VEC;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) *reinterpret_cast<V *>(dst + i * plane) = p[i];
+}
+
+// ---- dX = col2im(B dT B^T) (+ ReLU mask) ----------------------------------------------------------
+// Along one axis, pixel y lies in tile y/2 and in one neighbour; with patch offset r = y + 1 - 2*tile,
+// (B dT B^T)[r][.] = sum_u BT[u][r] dT[u][.], BT = [[1,0,-1,0],[0,1,1,0],[0,-1,1,0],[0,1,0,-1]]:
+//   r=0: +u0        r=1: +u1 -u2 +u3        r=2: -u0 +u1 +u2        r=3: -u3
+struct AxisTerms {
+    int tile[4], u[4];
+    float sign[4];  // 0 marks a term outside the tile grid
+};
+__device__ __forceinline__ AxisTerms axis_terms(int y, int n_tiles)
+{
+    AxisTerms o;
+    const int t = y >> 1;
+    if (y & 1) {  // r = 2 in tile t, r = 0 in tile t+1
+        o.tile[0] = t; o.u[0] = 0; o.sign[0] = -1.f;
+        o.tile[1] = t; o.u[1] = 1; o.sign[1] = 1.f;
+        o.tile[2] = t; o.u[2] = 2; o.sign[2] = 1.f;
+        const bool ok = t + 1 < n_tiles;
+        o.tile[3] = ok ? t + 1 : t; o.u[3] = 0; o.sign[3] = ok ? 1.f : 0.f;
+    } else {      // r = 1 in tile t, r = 3 in tile t-1
+        o.tile[0] = t; o.u[0] = 1; o.sign[0] = 1.f;
+        o.tile[1] = t; o.u[1] = 2; o.sign[1] = -1.f;
+        o.tile[2] = t; o.u[2] = 3; o.sign[2] = 1.f;
+        const bool ok = t >= 1;
+        o.tile[3] = ok ? t - 1 : t; o.u[3] = 3; o.sign[3] = ok ? -1.f : 0.f;
+    }
+    return o;
+}
+
+template <int VEC, bool MASK>
+__global__ __launch_bounds__(256) void imtrans_grad_kernel(const float *__restrict__ dT, const float *__restrict__ mask_src,
+                                                           float *__restrict__ dX, int H, int W, int C, int nH, int nW,
+                                                           unsigned items, size_t plane)
+{
+    using V = typename GVec<VEC>::type;
+    const unsigned idx = xcd_swizzle(blockIdx.x, gridDim.x) * 256 + threadIdx.x;
+    if (idx >= items) return;
+    const unsigned CV = C / VEC;
+    const unsigned cv = idx % CV;
+    unsigned p = idx / CV;
+    const int x = p % W;
+    p /= W;
+    const int y = p % H;
+    const unsigned b = p / H;
+    const AxisTerms ry = axis_terms(y, nH), rx = axis_terms(x, nW);
+    float acc[VEC];
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float sg = ry.sign[i] * rx.sign[j];
+            const size_t off = static_cast<size_t>(4 * ry.u[i] + rx.u[j]) * plane +
+                               ((static_cast<size_t>(b) * nH + ry.tile[i]) * nW + rx.tile[j]) * C + static_cast<size_t>(cv) * VEC;
+            const V g = *reinterpret_cast<const V *>(dT + off);
+            const float *gp = reinterpret_cast<const float *>(&g);
+            if (MASK) {
+                const V t = *reinterpret_cast<const V *>(mask_src + off);
+                const float *tp = reinterpret_cast<const float *>(&t);
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) acc[q] += (sg != 0.f && tp[q] > 0.f) ? sg * gp[q] : 0.f;
+            } else {
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) acc[q] += sg != 0.f ? sg * gp[q] : 0.f;
+            }
+        }
+    float *o = dX + static_cast<size_t>(idx) * VEC;
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) o[q] = acc[q];
+}
+
+// ---- rocBLAS handle: one per host thread and device, created on first use -------------------------
+rocblas_handle blas_handle()
+{
+    constexpr int kMaxDevices = 64;
+    static thread_local rocblas_handle handles[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    if (handles[dev] == nullptr && rocblas_create_handle(&handles[dev]) != rocblas_status_success) handles[dev] = nullptr;
+    return handles[dev];
+}
+
+}  // namespace
+}  // namespace swc
+
+extern "C" int swc_winograd2x2_conv_grad(const float *TInput, const float *Weight, const float *Output_grad,
+                                         float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,
+                                         long long *tmp_ptr_buffer, int C, int B, int H, int W, int K, int pad_h,
+                                         int pad_w, swc_stream_t stream)
+{
+    using namespace swc;
+    (void)tmp_ptr_buffer;
+    if (TInput == nullptr || Weight == nullptr || Output_grad == nullptr || TInput_grad == nullptr ||
+        Weight_grad == nullptr || tmp_data_buffer == nullptr)
+        return SWC_ERR_NULL_POINTER;
+    if (C <= 0 || B <= 0 || H <= 0 || W <= 0 || K <= 0 || (H & 1) || (W & 1)) return SWC_ERR_BAD_DIMS;  // H = 2nH, W = 2nW
+    if (pad_h != 1 || pad_w != 1) return SWC_ERR_BAD_PAD;
+    const int nH = H / 2, nW = W / 2;
+    const size_t M = static_cast<size_t>(B) * nH * nW;
+    if (M >= (1ull << 31) || M * K >= (1ull << 32) || M * C >= (1ull << 40)) return SWC_ERR_BAD_DIMS;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+
+    const bool vec = (K % 4 == 0) && aligned16(Output_grad) && aligned16(tmp_data_buffer);
+    const unsigned items = static_cast<unsigned>(M * (vec ? K / 4 : K));
+    const dim3 grid((items + 255) / 256), block(256);
+    if (vec)
+        output_transform_grad_kernel<4><<<grid, block, 0, s>>>(Output_grad, tmp_data_buffer, nW, K, items, M * K);
+    else
+        output_transform_grad_kernel<1><<<grid, block, 0, s>>>(Output_grad, tmp_data_buffer, nW, K, items, M * K);
+    int st = check_launch();
+    if (st != SWC_OK) return st;
+
+    rocblas_handle h = blas_handle();
+    if (h == nullptr || rocblas_set_stream(h, s) != rocblas_status_success) return SWC_ERR_HIP;
+    const float one = 1.f, zero = 0.f;
+    const int Mi = static_cast<int>(M);
+    // Row-major dTI[i] (M x C) = dP[i] (M x K) . W[i]^T, as column-major (C x M) = op_T(W: K x C) . (dP: K x M):
+    // the call at winograd2x2_conv_grad_cuda.cu.cc:103-108.
+    rocblas_status rs = rocblas_sgemm_strided_batched(h, rocblas_operation_transpose, rocblas_operation_none, C, Mi, K, &one,
+                                                      Weight, K, static_cast<rocblas_stride>(C) * K, tmp_data_buffer, K,
+                                                      static_cast<rocblas_stride>(M) * K, &zero, TInput_grad, C,
+                                                      static_cast<rocblas_stride>(M) * C, 16);
+    if (rs != rocblas_status_success) return SWC_ERR_HIP;
+    // Row-major dW[i] (C x K) = TI[i]^T . dP[i], as column-major (K x C) = (dP: K x M) . op_T(TI: C x M):
+    // the call at winograd2x2_conv_grad_cuda.cu.cc:115-120.
+    rs = rocblas_sgemm_strided_batched(h, rocblas_operation_none, rocblas_operation_transpose, K, C, Mi, &one,
+                                       tmp_data_buffer, K, static_cast<rocblas_stride>(M) * K, TInput, C,
+                                       static_cast<rocblas_stride>(M) * C, &zero, Weight_grad, K,
+                                       static_cast<rocblas_stride>(C) * K, 16);
+    return rs == rocblas_status_success ? SWC_OK : SWC_ERR_HIP;
+}
+
+extern "C" int swc_winograd2x2_imtrans_grad(const float *TransIm_grad, const float *relu_mask_source, float *Input_grad,
+                                            int C, int B, int H, int W, int pad_h, int pad_w, swc_stream_t stream)
+{
+    using namespace swc;
+    if (TransIm_grad == nullptr || Input_grad == nullptr) return SWC_ERR_NULL_POINTER;
+    if (C <= 0 || B <= 0 || H <= 0 || W <= 0) return SWC_ERR_BAD_DIMS;
+    if (pad_h != 1 || pad_w != 1) return SWC_ERR_BAD_PAD;
+    const int nH = (H + 1) / 2, nW = (W + 1) / 2;
+    const size_t pixels = static_cast<size_t>(B) * H * W;
+    if (pixels * C >= (1ull << 32)) return SWC_ERR_BAD_DIMS;
+    const size_t plane = static_cast<size_t>(B) * nH * nW * C;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool vec = (C % 4 == 0) && aligned16(TransIm_grad) && aligned16(Input_grad) &&
+                     (relu_mask_source == nullptr || aligned16(relu_mask_source));
+    const unsigned items = static_cast<unsigned>(pixels * (vec ? C / 4 : C));
+    const dim3 grid((items + 255) / 256), block(256);
+#define SWC_LAUNCH(VEC, MASK)                                                                                        \
+    imtrans_grad_kernel<VEC, MASK><<<grid, block, 0, s>>>(TransIm_grad, relu_mask_source, Input_grad, H, W, C, nH, nW, \
+                                                          items, plane)
+    if (vec) {
+        if (relu_mask_source) SWC_LAUNCH(4, true); else SWC_LAUNCH(4, false);
+    } else {
+        if (relu_mask_source) SWC_LAUNCH(1, true); else SWC_LAUNCH(1, false);
+    }
+#undef SWC_LAUNCH
+    return check_launch();
+}
+
+void Winograd2x2ConvGradComputeLauncher(const float *TInput, const float *Weight, const float *Output_grad,
+                                        float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,
+                                        long long *tmp_ptr_buffer, int C, int B, int H, int W, int K, int pad_h, int pad_w)
+{
+    const int st = swc_winograd2x2_conv_grad(TInput, Weight, Output_grad, TInput_grad, Weight_grad, tmp_data_buffer,
+                                             tmp_ptr_buffer, C, B, H, W, K, pad_h, pad_w, nullptr);
+    if (st != SWC_OK) std::fprintf(stderr, "Winograd2x2ConvGradComputeLauncher: %s\n", swc_strerror(st));
+}
+
+void Winograd2x2ImTransGradComputeLauncher(const float *Output_grad, float *Input_grad, int C, int B, int H, int W,
+                                           int pad_h, int pad_w)
+{
+    const int st = swc_winograd2x2_imtrans_grad(Output_grad, nullptr, Input_grad, C, B, H, W, pad_h, pad_w, nullptr);
+    if (st != SWC_OK) std::fprintf(stderr, "Winograd2x2ImTransGradComputeLauncher: %s\n", swc_strerror(st));
+}

@@ -23,11 +23,14 @@ C_SYMBOLS = (
     "swc_winograd2x2_imtrans", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
+    "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad",
 )
 # The two C++-linkage launchers with the reference's exact signatures (Itanium mangling).
 CXX_SYMBOLS = (
     "_Z33Winograd2x2ImTransComputeLauncherPKfPfiiiiii",
     "_Z30Winograd2x2ConvComputeLauncherPKfS0_PfS1_PKxiiiiiii",
+    "_Z34Winograd2x2ConvGradComputeLauncherPKfS0_S0_PfS1_S1_Pxiiiiiii",
+    "_Z37Winograd2x2ImTransGradComputeLauncherPKfPfiiiiii",
 )
 
 _lib = None
@@ -77,6 +80,10 @@ def lib():
         L.swc_winograd2x2_conv_op_shape.argtypes = [i32, i64p, i32, i64p, i64p]
         L.swc_winograd2x2_conv_op_compute.restype = i32
         L.swc_winograd2x2_conv_op_compute.argtypes = [fp, i32, i64p, fp, i32, i64p, fp, i32, i64p, i32, vp]
+        L.swc_winograd2x2_conv_grad.restype = i32
+        L.swc_winograd2x2_conv_grad.argtypes = [fp] * 7 + [i32] * 7 + [vp]
+        L.swc_winograd2x2_imtrans_grad.restype = i32
+        L.swc_winograd2x2_imtrans_grad.argtypes = [fp] * 3 + [i32] * 6 + [vp]
         _lib = L
     return _lib
 
@@ -104,7 +111,4 @@ def require_cuda_f32(t, name, rank):
         # The reference's CPU kernels print a message and exit(-1)
         # (winograd2x2_imTrans_op.cc:82-83, winograd2x2_conv_op.cc:89-90); here it is an error.
         raise RuntimeError("%s is on %s: these ops run on the GPU only (no CPU kernel exists)" % (name, t.device))
-    if torch.is_grad_enabled() and t.requires_grad:
-        raise NotImplementedError(
-            "%s requires grad: only the forward ops are implemented; wrap the call in torch.no_grad()" % name)
     return t.contiguous()

@@ -2,7 +2,8 @@
 
 Mirrors winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv.py of the reference:
 ``winograd2x2_conv(I, W)`` (:13-14) with the shape rule of its RegisterShape function
-(:19-29).  The gradient registration (:31-36) has no counterpart: forward only.
+(:19-29), ``winograd2x2_conv_grad(i1, i2, grad)`` (:16-17), and the gradient registration
+(:31-36) as a torch.autograd.Function.
 """
 import os
 import sys
@@ -23,11 +24,7 @@ def winograd2x2_conv_shape(i_shape, w_shape):
     return tuple(out)
 
 
-def winograd2x2_conv(I, W, precision="fp32", out=None):
-    """I: [16,B,nH,nW,C], W: [16,C,K], float32 on the GPU -> [B,2nH,2nW,K] (uncropped).
-
-    ``precision="bf16"`` rounds both GEMM operands to bf16 (fp32 accumulate).
-    """
+def _forward(I, W, precision, out):
     if precision not in PRECISIONS:
         raise ValueError("precision must be one of %s" % sorted(PRECISIONS))
     I = swc_hip.require_cuda_f32(I, "I", 5)
@@ -47,3 +44,52 @@ def winograd2x2_conv(I, W, precision="fp32", out=None):
             out.data_ptr(), 4, swc_hip.dims(out.shape), PRECISIONS[precision], stream)
     swc_hip.check(st, "winograd2x2_conv")
     return out
+
+
+def winograd2x2_conv_grad(i1, i2, grad):
+    """(I [16,B,nH,nW,C], W [16,C,K], grad [B,2nH,2nW,K]) -> (dI, dW), as the reference's
+    winograd2x2_conv_grad (winograd2x2_conv.py:16-17).  fp32 throughout."""
+    I = swc_hip.require_cuda_f32(i1, "i1", 5)
+    W = swc_hip.require_cuda_f32(i2, "i2", 3)
+    grad = swc_hip.require_cuda_f32(grad, "grad", 4)
+    want = winograd2x2_conv_shape(I.shape, W.shape)
+    if tuple(grad.shape) != want:
+        raise ValueError("grad must have shape %s, got %s" % (want, tuple(grad.shape)))
+    _, B, nH, nW, C = I.shape
+    K = W.shape[2]
+    dI, dW = torch.empty_like(I), torch.empty_like(W)
+    tmp = torch.empty(16 * B * nH * nW * K, dtype=torch.float32, device=I.device)  # as winograd2x2_conv_grad_op.cc:69-71
+    with torch.cuda.device(I.device):
+        st = swc_hip.lib().swc_winograd2x2_conv_grad(
+            I.data_ptr(), W.data_ptr(), grad.data_ptr(), dI.data_ptr(), dW.data_ptr(), tmp.data_ptr(), None,
+            C, B, 2 * nH, 2 * nW, K, 1, 1, torch.cuda.current_stream().cuda_stream)
+    swc_hip.check(st, "winograd2x2_conv_grad")
+    return dI, dW
+
+
+class _ConvFunction(torch.autograd.Function):
+    """The RegisterGradient hook of the reference (winograd2x2_conv.py:31-36).  The backward is fp32
+    whatever the forward's GEMM precision was."""
+
+    @staticmethod
+    def forward(ctx, I, W, precision):
+        ctx.save_for_backward(I, W)
+        return _forward(I, W, precision, None)
+
+    @staticmethod
+    def backward(ctx, grad):
+        I, W = ctx.saved_tensors
+        dI, dW = winograd2x2_conv_grad(I, W, grad.contiguous())
+        return dI, dW, None
+
+
+def winograd2x2_conv(I, W, precision="fp32", out=None):
+    """I: [16,B,nH,nW,C], W: [16,C,K], float32 on the GPU -> [B,2nH,2nW,K] (uncropped).
+
+    ``precision="bf16"`` rounds both GEMM operands to bf16 (fp32 accumulate).  Differentiable
+    through ``winograd2x2_conv_grad`` when an input requires grad.
+    """
+    needs_grad = torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (I, W))
+    if out is None and needs_grad:
+        return _ConvFunction.apply(I, W, precision)
+    return _forward(I, W, precision, out)

@@ -2,7 +2,8 @@
 
 Mirrors winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans.py of the reference:
 ``winograd2x2_imTrans(I)`` (:13-14) with the shape rule of its RegisterShape function
-(:20-27).  The gradient registration (:29-33) has no counterpart: forward only.
+(:20-27), ``winograd2x2_imTrans_grad(grad)`` (:16-17), and the gradient registration (:29-33)
+as a torch.autograd.Function.
 """
 import os
 import sys
@@ -21,13 +22,7 @@ def winograd2x2_imTrans_shape(shape):
     return tuple(out)
 
 
-def winograd2x2_imTrans(I, relu=False, out=None):
-    """I: [B,H,W,C] float32 NHWC on the GPU -> [16,B,nH,nW,C].
-
-    ``relu=True`` applies the Winograd-domain ReLU inside the same kernel (what
-    ``nl(winograd2x2_imTrans(x))`` with ``nl=tf.nn.relu`` computes in
-    ResNet-18-var/winograd_imtrans.py:16-17).  ``out`` may supply the result tensor.
-    """
+def _forward(I, relu, out):
     I = swc_hip.require_cuda_f32(I, "I", 4)
     shape = winograd2x2_imTrans_shape(I.shape)
     if out is None:
@@ -41,3 +36,63 @@ def winograd2x2_imTrans(I, relu=False, out=None):
             I.data_ptr(), 4, swc_hip.dims(I.shape), out.data_ptr(), 5, swc_hip.dims(out.shape), int(bool(relu)), stream)
     swc_hip.check(st, "winograd2x2_imTrans")
     return out
+
+
+def winograd2x2_imTrans_grad(grad, H=None, W=None, relu_output=None):
+    """grad: [16,B,nH,nW,C] -> gradient w.r.t. the op's input, [B,H,W,C].
+
+    As in the reference (winograd2x2_imTrans_grad_op.cc:44-45) H and W default to 2*nH, 2*nW.
+    ``relu_output``: the forward result computed with ``relu=True``; the gradient is then taken
+    through the fused ReLU.  ``grad`` is left untouched (the reference overwrites it).
+    """
+    grad = swc_hip.require_cuda_f32(grad, "grad", 5)
+    if grad.shape[0] != 16:
+        raise ValueError("grad must have shape [16,B,nH,nW,C]")
+    _, B, nH, nW, C = grad.shape
+    H = 2 * nH if H is None else int(H)
+    W = 2 * nW if W is None else int(W)
+    if (H + 1) // 2 != nH or (W + 1) // 2 != nW:
+        raise ValueError("H, W = %d, %d do not tile into %d x %d" % (H, W, nH, nW))
+    mask_ptr = None
+    if relu_output is not None:
+        relu_output = swc_hip.require_cuda_f32(relu_output, "relu_output", 5)
+        if relu_output.shape != grad.shape:
+            raise ValueError("relu_output must have grad's shape")
+        mask_ptr = relu_output.data_ptr()
+    out = torch.empty((B, H, W, C), dtype=torch.float32, device=grad.device)
+    with torch.cuda.device(grad.device):
+        st = swc_hip.lib().swc_winograd2x2_imtrans_grad(grad.data_ptr(), mask_ptr, out.data_ptr(), C, B, H, W, 1, 1,
+                                                        torch.cuda.current_stream().cuda_stream)
+    swc_hip.check(st, "winograd2x2_imTrans_grad")
+    return out
+
+
+class _ImTransFunction(torch.autograd.Function):
+    """The RegisterGradient hook of the reference (winograd2x2_imTrans.py:29-33), with the fused ReLU."""
+
+    @staticmethod
+    def forward(ctx, I, relu):
+        out = _forward(I, relu, None)
+        ctx.hw = (I.shape[1], I.shape[2])
+        ctx.relu = bool(relu)
+        if relu:
+            ctx.save_for_backward(out)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        relu_output = ctx.saved_tensors[0] if ctx.relu else None
+        return winograd2x2_imTrans_grad(grad.contiguous(), ctx.hw[0], ctx.hw[1], relu_output), None
+
+
+def winograd2x2_imTrans(I, relu=False, out=None):
+    """I: [B,H,W,C] float32 NHWC on the GPU -> [16,B,nH,nW,C].
+
+    ``relu=True`` applies the Winograd-domain ReLU inside the same kernel (what
+    ``nl(winograd2x2_imTrans(x))`` with ``nl=tf.nn.relu`` computes in
+    ResNet-18-var/winograd_imtrans.py:16-17).  ``out`` may supply the result tensor (forward only).
+    Differentiable: gradients flow through ``winograd2x2_imTrans_grad``.
+    """
+    if out is None and isinstance(I, torch.Tensor) and I.requires_grad and torch.is_grad_enabled():
+        return _ImTransFunction.apply(I, relu)
+    return _forward(I, relu, out)

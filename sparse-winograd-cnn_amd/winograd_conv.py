@@ -23,10 +23,11 @@ class WinogradConv(torch.nn.Module):
       std = sqrt(1.3*factor/fan_in), fan_in = 16*in_channel as TensorFlow 1.x computes
       it for a rank-3 shape.
     * ``mask``: optional 0/1 array of the weight's shape; the reference multiplies it in on
-      every step (:23-25).  Here the product W*mask is cached and refreshed by
-      ``refresh()`` after W changes.
+      every step (:23-25).  Here W*mask is recomputed only while gradients are being recorded
+      (so that they flow to W through the mask); otherwise the product is cached and refreshed
+      by ``refresh()`` after W changes.
 
-    Forward only: W carries no gradient.
+    W is a trainable parameter; gradients come from ``winograd2x2_conv_grad``.
     """
 
     def __init__(self, in_channel, out_channel, mask=None, W_init=None, precision="fp32", device=None):
@@ -40,7 +41,7 @@ class WinogradConv(torch.nn.Module):
             W_init(W)
         else:
             W.copy_(torch.as_tensor(W_init, dtype=torch.float32).reshape(W.shape))
-        self.W = torch.nn.Parameter(W, requires_grad=False)
+        self.W = torch.nn.Parameter(W)
         if mask is not None:
             mask = torch.as_tensor(mask, dtype=torch.float32, device=W.device).reshape(W.shape).clone()
         self.register_buffer("mask", mask)
@@ -58,4 +59,8 @@ class WinogradConv(torch.nn.Module):
         return self._masked
 
     def forward(self, x):
-        return winograd2x2_conv.winograd2x2_conv.winograd2x2_conv(x, self.masked_weight(), precision=self.precision)
+        if torch.is_grad_enabled() and self.W.requires_grad:
+            w = self.W if self.mask is None else self.W * self.mask
+        else:
+            w = self.masked_weight()
+        return winograd2x2_conv.winograd2x2_conv.winograd2x2_conv(x, w, precision=self.precision)

@@ -314,5 +314,5 @@ def test_layer_wrappers_on_gpu(oracle, dev):
     assert np.array_equal(WinogradImTrans(xd).cpu().numpy(), oracle.imtrans(x))
     assert np.array_equal(WinogradImTrans(xd, torch.tanh).cpu().numpy(),
                           torch.tanh(gpu(oracle.imtrans(x), dev)).cpu().numpy())
-    y = layer(WinogradImTrans(xd, torch.relu)).cpu().numpy()
+    y = layer(WinogradImTrans(xd, torch.relu)).detach().cpu().numpy()
     assert rel_max(y, oracle.conv(oracle.imtrans(x, relu=True), w * mask, acc64=True)) <= TOL

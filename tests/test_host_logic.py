@@ -20,7 +20,8 @@ def test_library_exports_every_declared_symbol():
     declared = set(re.findall(r"SWC_API\s+[\w\s\*]+?\b(swc_\w+|Winograd2x2\w+)\s*\(", header))
     assert set(swc_hip.C_SYMBOLS) == {d for d in declared if d.startswith("swc_")}
     assert {d for d in declared if d.startswith("Winograd2x2")} == {
-        "Winograd2x2ImTransComputeLauncher", "Winograd2x2ConvComputeLauncher"}
+        "Winograd2x2ImTransComputeLauncher", "Winograd2x2ConvComputeLauncher",
+        "Winograd2x2ConvGradComputeLauncher", "Winograd2x2ImTransGradComputeLauncher"}
     L = ctypes.CDLL(swc_hip.LIB_PATH)
     for name in swc_hip.C_SYMBOLS + swc_hip.CXX_SYMBOLS:
         assert getattr(L, name) is not None, name
@@ -88,6 +89,13 @@ def test_launchers_reject_bad_arguments_before_touching_the_gpu():
         assert conv(p, p, None, None, None, 4, 1, 2, 2, 4, 1, 1, None) == swc_hip.SWC_ERR_NULL_POINTER
         assert conv(p, p, p, None, None, 4, 1, 2, 2, 0, 1, 1, None) == swc_hip.SWC_ERR_BAD_DIMS
         assert conv(p, p, p, None, None, 4, 1, 2, 2, 4, 1, 0, None) == swc_hip.SWC_ERR_BAD_PAD
+    # gradient launchers
+    assert L.swc_winograd2x2_conv_grad(p, p, p, p, p, None, None, 4, 1, 4, 4, 4, 1, 1, None) == swc_hip.SWC_ERR_NULL_POINTER
+    assert L.swc_winograd2x2_conv_grad(p, p, p, p, p, p, None, 4, 1, 5, 4, 4, 1, 1, None) == swc_hip.SWC_ERR_BAD_DIMS  # H odd
+    assert L.swc_winograd2x2_conv_grad(p, p, p, p, p, p, None, 4, 1, 4, 4, 4, 2, 1, None) == swc_hip.SWC_ERR_BAD_PAD
+    assert L.swc_winograd2x2_imtrans_grad(None, None, p, 4, 1, 4, 4, 1, 1, None) == swc_hip.SWC_ERR_NULL_POINTER
+    assert L.swc_winograd2x2_imtrans_grad(p, None, p, 4, 0, 4, 4, 1, 1, None) == swc_hip.SWC_ERR_BAD_DIMS
+    assert L.swc_winograd2x2_imtrans_grad(p, None, p, 4, 1, 4, 4, 1, 0, None) == swc_hip.SWC_ERR_BAD_PAD
     # op level: an output of the wrong shape is refused
     i4, o5 = swc_hip.dims((1, 4, 4, 4)), swc_hip.dims((16, 1, 2, 2, 5))
     assert L.swc_winograd2x2_imtrans_op_compute(p, 4, i4, p, 5, o5, 0, None) == swc_hip.SWC_ERR_BAD_DIMS
@@ -125,7 +133,7 @@ def test_layer_wrappers_signatures():
     assert inspect.signature(WinogradImTrans).parameters["nl"].default is identity
     assert list(inspect.signature(WinogradConv.__init__).parameters)[1:5] == ["in_channel", "out_channel", "mask", "W_init"]
     layer = WinogradConv(8, 12)
-    assert tuple(layer.W.shape) == (16, 8, 12) and not layer.W.requires_grad
+    assert tuple(layer.W.shape) == (16, 8, 12) and layer.W.requires_grad
     std = float(layer.W.std())
     assert 0 < std < np.sqrt(1.3 * (2 * 9 / 32) / (16 * 8))
     mask = np.zeros((16, 8, 12), dtype=np.float32)
