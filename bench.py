@@ -235,6 +235,12 @@ def main():
         f_imtrans()
         f_conv()
 
+    fused_ok = args.precision == "fp32" and L.swc_winograd2x2_relu_conv(xp, wp, yp, C, B, H, W, K, 1, 1, 1, stream) == 0
+
+    def f_fused():
+        if L.swc_winograd2x2_relu_conv(xp, wp, yp, C, B, H, W, K, 1, 1, 1, stream) != 0:
+            raise RuntimeError("swc_winograd2x2_relu_conv failed")
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -248,6 +254,10 @@ def main():
     ms_imtrans = time_loop(f_imtrans, args.steps, torch)
     ms_conv = time_loop(f_conv, args.steps, torch)
     ms_pair = time_loop(step, args.steps, torch)
+    ms_fused = time_loop(f_fused, args.steps, torch) if fused_ok else None
+    if fused_ok:
+        y_fused = y.clone()
+        step()  # leave the two-op result in y for the parity gate
     torch.cuda.synchronize()
 
     direct_flops = 18.0 * B * H * W * C * K
@@ -297,6 +307,15 @@ def main():
         "ms_conv": round(ms_conv, 5),
         "ms_pair_events": round(ms_pair, 5),
         "roofline": conv_roofline,
+        # the same layer as one kernel (swc_winograd2x2_relu_conv): TI never reaches memory
+        "fused_layer": None if not fused_ok else {
+            "ms": round(ms_fused, 5),
+            "effective_direct_conv_GFLOPs": round(direct_flops / (ms_fused * 1e-3) / 1e9, 1),
+            "mfma_TFLOPs": round(gemm_flops / (ms_fused * 1e-3) / 1e12, 2),
+            "mfma_frac": round(gemm_flops / (ms_fused * 1e-3) / 1e12 / FP32_MFMA_PEAK_TF, 4),
+            "algorithmic_bytes_per_launch": 4.0 * B * H * W * C + 64.0 * C * K + 16.0 * M * K,
+            "max_abs_diff_vs_two_op": float((y_fused - y).abs().max()),
+        },
         "roofline_imtrans": {
             "kernel": "winograd2x2_imTrans + ReLU",
             "bound": "hbm",

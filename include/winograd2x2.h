@@ -30,6 +30,7 @@ typedef void *swc_stream_t;
 #define SWC_ERR_BAD_PAD (-3)      /* pad_h/pad_w other than 1: the only geometry the ops define */
 #define SWC_ERR_HIP (-4)          /* the HIP runtime refused the launch; see swc_last_hip_error() */
 #define SWC_ERR_BAD_RANK (-5)     /* op-level wrappers: wrong tensor rank or leading dimension */
+#define SWC_ERR_UNSUPPORTED (-6)  /* valid arguments that this entry point has no kernel for (see its comment) */
 
 SWC_API const char *swc_strerror(int status);
 /* hipError_t of the most recent failed launch on the calling thread (0 if none). */
@@ -130,6 +131,24 @@ SWC_API int swc_winograd2x2_conv_op_compute(const float *input, int in_rank, con
                                     const float *weight, int w_rank, const int64_t *w_dims,
                                     float *output, int out_rank, const int64_t *out_dims,
                                     int precision, swc_stream_t stream);
+
+/*
+ * The layer pair in one kernel: swc_winograd2x2_imtrans(relu) followed by swc_winograd2x2_conv,
+ * without the [16,B,nH,nW,C] intermediate ever reaching memory.
+ *   Input [B,H,W,C], Weight [16,C,K]  ->  Output [B,2nH,2nW,K]   (fp32)
+ * No single counterpart in the reference: it is the composition of its two launchers and the
+ * tf.nn.relu between them, as the model applies them
+ * (ResNet-18-var/imagenet-resnet-transWino-prune.py:118-119; winograd_imtrans.py:16-17;
+ * winograd_conv.py:28).  The transformed activations are bit-identical to the stand-alone
+ * transform's, and the products are folded in the same ascending order, so the result agrees with
+ * the two-call sequence to GEMM rounding.
+ * Needs C % 8 == 0, K % 4 == 0, Weight 16-byte and Input 8-byte aligned, and fewer than 2^30 input
+ * elements; otherwise returns SWC_ERR_UNSUPPORTED and the caller uses the two entry points above
+ * (which need the intermediate buffer this one has no room for).
+ */
+SWC_API int swc_winograd2x2_relu_conv(const float *Input, const float *Weight, float *Output,
+                                      int C, int B, int H, int W, int K, int pad_h, int pad_w,
+                                      int relu, swc_stream_t stream);
 
 /* ---------------------------------------------------------------------------
  * Backward ops.

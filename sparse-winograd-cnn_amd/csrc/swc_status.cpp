@@ -22,6 +22,7 @@ extern "C" const char *swc_strerror(int status)
         case SWC_ERR_BAD_PAD: return "pad_h and pad_w must both be 1";
         case SWC_ERR_HIP: return "the HIP runtime refused the launch (see swc_last_hip_error)";
         case SWC_ERR_BAD_RANK: return "wrong tensor rank or leading dimension";
+        case SWC_ERR_UNSUPPORTED: return "this entry point has no kernel for these (valid) arguments";
         default: return "unknown status";
     }
 }

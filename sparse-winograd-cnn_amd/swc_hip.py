@@ -16,6 +16,7 @@ SWC_ERR_BAD_DIMS = -2
 SWC_ERR_BAD_PAD = -3
 SWC_ERR_HIP = -4
 SWC_ERR_BAD_RANK = -5
+SWC_ERR_UNSUPPORTED = -6
 
 # Every symbol include/winograd2x2.h declares with C linkage.
 C_SYMBOLS = (
@@ -23,7 +24,7 @@ C_SYMBOLS = (
     "swc_winograd2x2_imtrans", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
-    "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad",
+    "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad", "swc_winograd2x2_relu_conv",
 )
 # The two C++-linkage launchers with the reference's exact signatures (Itanium mangling).
 CXX_SYMBOLS = (
@@ -80,6 +81,8 @@ def lib():
         L.swc_winograd2x2_conv_op_shape.argtypes = [i32, i64p, i32, i64p, i64p]
         L.swc_winograd2x2_conv_op_compute.restype = i32
         L.swc_winograd2x2_conv_op_compute.argtypes = [fp, i32, i64p, fp, i32, i64p, fp, i32, i64p, i32, vp]
+        L.swc_winograd2x2_relu_conv.restype = i32
+        L.swc_winograd2x2_relu_conv.argtypes = [fp] * 3 + [i32] * 8 + [vp]
         L.swc_winograd2x2_conv_grad.restype = i32
         L.swc_winograd2x2_conv_grad.argtypes = [fp] * 7 + [i32] * 7 + [vp]
         L.swc_winograd2x2_imtrans_grad.restype = i32

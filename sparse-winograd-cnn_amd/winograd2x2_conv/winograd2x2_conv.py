@@ -93,3 +93,34 @@ def winograd2x2_conv(I, W, precision="fp32", out=None):
     if out is None and needs_grad:
         return _ConvFunction.apply(I, W, precision)
     return _forward(I, W, precision, out)
+
+
+def winograd2x2_relu_conv(X, W, relu=True, out=None):
+    """The layer pair in one kernel: ``winograd2x2_conv(relu(winograd2x2_imTrans(X)), W)``.
+
+    X: [B,H,W,C] NHWC, W: [16,C,K], float32 on the GPU -> [B,2nH,2nW,K] (uncropped), fp32.  The
+    [16,B,nH,nW,C] intermediate is never materialised.  Shapes the fused kernel does not cover
+    (C % 8 != 0, K % 4 != 0, ...) run the two ops back to back instead.  Forward only.
+    """
+    import winograd2x2_imTrans.winograd2x2_imTrans as _it
+
+    X = swc_hip.require_cuda_f32(X, "X", 4)
+    W = swc_hip.require_cuda_f32(W, "W", 3)
+    if W.device != X.device:
+        raise ValueError("X and W must be on the same device")
+    B, H, Wd, C = X.shape
+    if W.shape[0] != 16 or W.shape[1] != C:
+        raise ValueError("W must have shape [16,%d,K], got %s" % (C, tuple(W.shape)))
+    K = W.shape[2]
+    shape = (B, 2 * ((H + 1) // 2), 2 * ((Wd + 1) // 2), K)
+    if out is None:
+        out = torch.empty(shape, dtype=torch.float32, device=X.device)
+    elif tuple(out.shape) != shape or out.dtype != torch.float32 or out.device != X.device or not out.is_contiguous():
+        raise ValueError("out must be a contiguous float32 tensor of shape %s on %s" % (shape, X.device))
+    with torch.cuda.device(X.device):
+        st = swc_hip.lib().swc_winograd2x2_relu_conv(X.data_ptr(), W.data_ptr(), out.data_ptr(), C, B, H, Wd, K, 1, 1,
+                                                     int(bool(relu)), torch.cuda.current_stream().cuda_stream)
+    if st == swc_hip.SWC_ERR_UNSUPPORTED:
+        return _forward(_it.winograd2x2_imTrans(X, relu=relu), W, "fp32", out)
+    swc_hip.check(st, "winograd2x2_relu_conv")
+    return out
