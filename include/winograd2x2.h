@@ -37,6 +37,12 @@ SWC_API const char *swc_strerror(int status);
 SWC_API int swc_last_hip_error(void);
 /* Library version, "major.minor". */
 SWC_API const char *swc_version(void);
+/* Diagnostic with no counterpart in the reference: the name of the convolution kernel that the calling
+ * thread's last swc_winograd2x2_conv / _conv_bf16 call launched ("" before the first): "sync" (any shape
+ * and alignment), "ring32" / "ring16" (64x64 tiles, 32- / 16-channel steps), "tall16" / "short16" (row
+ * groups of up to 112 / 32 rows, dealt evenly over the CUs).  Which one runs depends only on the shapes
+ * and pointer alignment; all give the same results to within the order of the reduction over C. */
+SWC_API const char *swc_winograd2x2_conv_last_kernel(void);
 
 /* ---------------------------------------------------------------------------
  * Launcher level: what the reference's TensorFlow op kernels call.

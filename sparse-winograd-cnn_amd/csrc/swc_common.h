@@ -10,6 +10,9 @@ namespace swc {
 // Records a failed HIP call for swc_last_hip_error() and maps it to SWC_ERR_HIP.
 int note_hip_error(hipError_t e);
 
+// Records which convolution kernel a call chose, for swc_winograd2x2_conv_last_kernel().
+void note_conv_kernel(const char *name);
+
 inline int check_launch()
 {
     hipError_t e = hipGetLastError();

@@ -4,7 +4,10 @@
 namespace swc {
 namespace {
 thread_local int g_last_hip_error = 0;
+thread_local const char *g_conv_kernel = "";
 }
+
+void note_conv_kernel(const char *name) { g_conv_kernel = name; }
 
 int note_hip_error(hipError_t e)
 {
@@ -28,5 +31,7 @@ extern "C" const char *swc_strerror(int status)
 }
 
 extern "C" int swc_last_hip_error(void) { return swc::g_last_hip_error; }
+
+extern "C" const char *swc_winograd2x2_conv_last_kernel(void) { return swc::g_conv_kernel; }
 
 extern "C" const char *swc_version(void) { return "0.1"; }

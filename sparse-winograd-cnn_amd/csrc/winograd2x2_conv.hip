@@ -48,17 +48,44 @@ bool async_eligible(const float *TI, const float *Wt, int C, int K)
            static_cast<size_t>(Cfg::BM) * C < (1ull << 29) && static_cast<size_t>(Cfg::BK) * K < (1ull << 29);
 }
 
+// rows_per_wg <= Cfg::BM rows of the [M,K] plane go to each workgroup.
 template <typename Cfg, int NSTAGE, bool BF16>
 int launch_async(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nH, int nW,
-                 hipStream_t stream)
+                 size_t rows_per_wg, hipStream_t stream)
 {
-    const size_t tiles_m = (M + Cfg::BM - 1) / Cfg::BM;
+    constexpr int lds_bytes = async_lds_bytes<Cfg, NSTAGE>();
+    static_assert(lds_bytes <= 64 * 1024, "larger tiles would need hipFuncAttributeMaxDynamicSharedMemorySize raised first");
+    const size_t tiles_m = (M + rows_per_wg - 1) / rows_per_wg;
     const size_t tiles_n = (static_cast<size_t>(K) + Cfg::BN - 1) / Cfg::BN;
     if (tiles_m * tiles_n >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
     const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n)), block(Cfg::NT);
-    conv_mfma_async_kernel<Cfg, NSTAGE, BF16><<<grid, block, 0, stream>>>(TI, Wt, Out, M, C, K, nH, nW,
-                                                                    static_cast<unsigned>(tiles_n));
+    conv_mfma_async_kernel<Cfg, NSTAGE, BF16><<<grid, block, lds_bytes, stream>>>(
+        TI, Wt, Out, M, C, K, nH, nW, static_cast<unsigned>(tiles_n), static_cast<unsigned>(rows_per_wg));
     return check_launch();
+}
+
+constexpr size_t kCUs = 256;  // MI355X
+
+// Passes the chip makes over `wgs` workgroups of equal length: the busiest CU sets the time, so whole
+// passes while the grid is small; with many short workgroups the tail evens out.
+double passes(size_t wgs)
+{
+    return wgs <= 8 * kCUs ? static_cast<double>((wgs + kCUs - 1) / kCUs) : static_cast<double>(wgs) / kCUs + 0.5;
+}
+
+// Rows per workgroup that split M into as many equal row groups as fill whole passes of the chip, but
+// never so few that one of the workgroup's 16-row MFMA tiles would hold no valid row at all (a
+// workgroup computes all of its tiles whatever their content).
+template <typename Cfg>
+size_t balanced_rows(size_t M, size_t tiles_n)
+{
+    const size_t groups_min = (M + Cfg::BM - 1) / Cfg::BM;
+    const size_t wgs = (groups_min * tiles_n + kCUs - 1) / kCUs * kCUs;
+    size_t groups = wgs / tiles_n;
+    if (groups < groups_min) groups = groups_min;
+    size_t rows = (M + groups - 1) / groups;
+    if (rows < static_cast<size_t>(Cfg::BM) - 15) rows = Cfg::BM - 15;
+    return rows < static_cast<size_t>(Cfg::BM) ? rows : static_cast<size_t>(Cfg::BM);
 }
 
 template <bool BF16>
@@ -71,14 +98,46 @@ int conv_entry(const float *Input, const float *Weight, float *Output, int C, in
     const size_t M = static_cast<size_t>(B) * nH * nW;
     if (M >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // 32x32 MFMAs, wave tile 32x32: the fewest LDS reads per MFMA; its results are bit-identical to
+    // the synchronous kernel's.
     using Tile32 = ConvCfg<64, 64, 32, 2, 2>;
     using Tile16 = ConvCfg<64, 64, 16, 2, 2>;
+    // 16x16 MFMAs, wave tile (16*TM)x16: row groups of any height up to 112 (Tall) or 32 (Short), so
+    // that M can be dealt evenly over the 256 CUs where 64-row tiles leave CUs idle or a ragged tail.
+    using Tall = ConvCfg<112, 64, 32, 1, 4, 2, 16>;
+    using Short = ConvCfg<32, 64, 64, 1, 4, 3, 16>;
+    if (!BF16) {
+        // Cost = passes x MFMA work of a wave per pass (in 16x16 tiles), weighted by what each kernel
+        // measured per unit of that work on MI355X relative to Tile32 (Tall 8 % more; Short about
+        // equal when its 64-channel steps are at least two per position, 15 % more otherwise).
+        const size_t tiles_n = (static_cast<size_t>(K) + 63) / 64;
+        const bool ok32 = async_eligible<Tile32>(Input, Weight, C, K);
+        const bool ok_tall = async_eligible<Tall>(Input, Weight, C, K);
+        const bool ok_short = async_eligible<Short>(Input, Weight, C, K);
+        const size_t rows_tall = balanced_rows<Tall>(M, tiles_n), rows_short = balanced_rows<Short>(M, tiles_n);
+        const double cost32 = ok32 ? passes((M + 63) / 64 * tiles_n) * 4.0 : 1e30;
+        const double cost_tall = ok_tall ? passes((M + rows_tall - 1) / rows_tall * tiles_n) * 7.0 * 1.08 : 1e30;
+        const double cost_short = ok_short ? passes((M + rows_short - 1) / rows_short * tiles_n) * 2.0 * (C >= 128 ? 0.98 : 1.15) : 1e30;
+        if (ok_tall && cost_tall < cost32 && cost_tall <= cost_short) {
+            note_conv_kernel("tall16");
+            return launch_async<Tall, 2, false>(Input, Weight, Output, M, C, K, nH, nW, rows_tall, s);
+        }
+        if (ok_short && cost_short < cost32) {
+            note_conv_kernel("short16");
+            return launch_async<Short, 2, false>(Input, Weight, Output, M, C, K, nH, nW, rows_short, s);
+        }
+    }
     // Ring depth: the fp32 step is long (16 MFMAs of 64 cycles per wave) and one tile in flight
     // covers the memory latency; the bf16 step is 8x shorter and needs two.
-    if (async_eligible<Tile32>(Input, Weight, C, K))
-        return launch_async<Tile32, BF16 ? 3 : 2, BF16>(Input, Weight, Output, M, C, K, nH, nW, s);
-    if (!BF16 && async_eligible<Tile16>(Input, Weight, C, K))
-        return launch_async<Tile16, 3, false>(Input, Weight, Output, M, C, K, nH, nW, s);
+    if (async_eligible<Tile32>(Input, Weight, C, K)) {
+        note_conv_kernel("ring32");
+        return launch_async<Tile32, BF16 ? 3 : 2, BF16>(Input, Weight, Output, M, C, K, nH, nW, Tile32::BM, s);
+    }
+    if (!BF16 && async_eligible<Tile16>(Input, Weight, C, K)) {
+        note_conv_kernel("ring16");
+        return launch_async<Tile16, 3, false>(Input, Weight, Output, M, C, K, nH, nW, Tile16::BM, s);
+    }
+    note_conv_kernel("sync");
     return launch_sync<Tile32, BF16>(Input, Weight, Output, M, C, K, nH, nW, s);
 }
 

@@ -10,6 +10,7 @@ namespace swc {
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -68,48 +69,57 @@ __device__ __forceinline__ float4 buffer_load_f4(__amdgpu_buffer_rsrc_t r, unsig
 
 constexpr unsigned kOutOfRange = 0xfffffff0u;  // a byte offset no descriptor here reaches
 
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int OCC_ = 2>
+// MF selects the MFMA shape of the asynchronous kernel: 32 = v_mfma_f32_32x32x2_f32 (16 accumulator
+// registers per tile), 16 = v_mfma_f32_16x16x4_f32 (4 registers per tile, 16-row granularity).
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int OCC_ = 2, int MF_ = 32>
 struct ConvCfg {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_, MF = MF_;
     static constexpr int OCC = OCC_;                     // waves per SIMD the register budget allows
     static constexpr int NT = WGM * WGN * 64;            // threads per workgroup
     static constexpr int WM = BM / WGM, WN = BN / WGN;   // wave tile
-    static constexpr int TM = WM / 32, TN = WN / 32;     // 32x32 MFMA tiles per wave
-    static constexpr int LDA = BK + 4;  // row stride (floats): 4*odd keeps b128 row reads conflict-free
+    static constexpr int TM = WM / MF, TN = WN / MF;     // MFMA tiles per wave
+    static constexpr int LG = 64 / MF;                   // lane groups: each feeds 4 reduction indices per operand read
+    static constexpr int KG = 4 * LG;                    // reduction indices per operand group (4 MFMAs)
+    static constexpr int REGS = MF * MF / 64;            // accumulator registers per tile
+    static constexpr int LDA = BK + 4;  // synchronous kernel: row stride (floats), 4*odd keeps b128 row reads conflict-free
     static constexpr int LDB = BN + 4;
-    static constexpr int NA = BM * BK / (4 * NT);        // float4 per thread per A tile
+    static constexpr int NA = BM * BK / (4 * NT);        // synchronous kernel: float4 per thread per A tile
     static constexpr int NB = BK * BN / (4 * NT);
-    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile is made of 32x32 MFMA tiles");
-    static_assert(BK % 8 == 0, "a k-step feeds 4 MFMAs from one b128 read per lane group");
-    static_assert((BK / 4) % 2 == 1 || BK % 8 == 0, "LDA");
-    static_assert(BM * BK % (4 * NT) == 0 && BK * BN % (4 * NT) == 0, "tile loads divide evenly");
+    static_assert(MF == 32 || MF == 16, "MFMA tile is 32x32 or 16x16");
+    static_assert(WM % MF == 0 && WN % MF == 0, "wave tile is made of whole MFMA tiles");
+    static_assert(BK % KG == 0, "a step is a whole number of operand groups");
 };
 
-// Scatter of the four output tiles: tile row m = (b*nH + th)*nW + tw -> pixels (2th+dy, 2tw+dx)
-// of image b (winograd2x2_conv_cuda.cu.cc:48-51).  Accumulator register r of lane (lg, li)
-// holds row 8*(r/4) + 4*lg + r%4 and column li of a 32x32 tile.  M < 2^31 (checked by the
-// launcher), so tile-row arithmetic fits 32 bits.
 template <typename Cfg>
-__device__ __forceinline__ void store_output(const floatx16 (&Y)[4][Cfg::TM][Cfg::TN], float *__restrict__ Out,
-                                             size_t M, int K, int nW, size_t m0, int n0, int wm0, int wn0, int li,
-                                             int lg)
+using AccT = typename std::conditional<Cfg::MF == 32, floatx16, floatx4>::type;
+
+// Scatter of the four output tiles: tile row m = (b*nH + th)*nW + tw -> pixels (2th+dy, 2tw+dx)
+// of image b (winograd2x2_conv_cuda.cu.cc:48-51).  Accumulator register r of lane (lg, li) holds
+// column li and row 8*(r/4) + 4*lg + r%4 of a 32x32 tile, row 4*lg + r of a 16x16 tile.  Only the
+// first rows_valid rows of the workgroup's tile are stored.  M < 2^31 (checked by the launcher),
+// so tile-row arithmetic fits 32 bits.
+template <typename Cfg>
+__device__ __forceinline__ void store_output(const AccT<Cfg> (&Y)[4][Cfg::TM][Cfg::TN], float *__restrict__ Out,
+                                             unsigned rows_valid, int K, int nW, size_t m0, int n0, int wm0, int wn0,
+                                             int li, int lg)
 {
-    constexpr int TM = Cfg::TM, TN = Cfg::TN;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, MF = Cfg::MF;
     const size_t oW = 2 * static_cast<size_t>(nW);
     const size_t row_stride = oW * K;
-    const unsigned M32 = static_cast<unsigned>(M), m032 = static_cast<unsigned>(m0);
+    const unsigned m032 = static_cast<unsigned>(m0);
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const unsigned gm = m032 + wm0 + tm * 32 + 8 * (r / 4) + 4 * lg + (r % 4);
-            if (gm >= M32) continue;
+        for (int r = 0; r < Cfg::REGS; ++r) {
+            const unsigned row = wm0 + tm * MF + (MF == 32 ? 8 * (r / 4) + 4 * lg + (r % 4) : 4 * lg + r);
+            if (row >= rows_valid) continue;
+            const unsigned gm = m032 + row;
             const unsigned bt = gm / static_cast<unsigned>(nW);  // b*nH + th
             const unsigned tw = gm - bt * static_cast<unsigned>(nW);
             float *o = Out + (static_cast<size_t>(bt) * 2 * oW + 2 * tw) * K;
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
-                const int col = n0 + wn0 + tn * 32 + li;
+                const int col = n0 + wn0 + tn * MF + li;
                 if (col >= K) continue;
                 o[col] = Y[0][tm][tn][r];
                 o[K + col] = Y[1][tm][tn][r];
@@ -134,6 +144,8 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, LDA = Cfg::LDA, LDB = Cfg::LDB, NA = Cfg::NA, NB = Cfg::NB;
     constexpr int KS = BK / 8;
+    static_assert(Cfg::MF == 32, "the register-staged kernel is written for 32x32 MFMA tiles");
+    static_assert(BM * BK % (4 * NT) == 0 && BK * BN % (4 * NT) == 0, "tile loads divide evenly");
 
     __shared__ __attribute__((aligned(16))) float As[2][BM * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
@@ -335,7 +347,7 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
                 for (int tn = 0; tn < TN; ++tn) asm volatile("" : "+v"(Y[j][tm][tn]));
     }
 
-    store_output<Cfg>(Y, Out, M, K, nW, m0, n0, wm0, wn0, li, lg);
+    store_output<Cfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -371,6 +383,13 @@ __device__ __forceinline__ unsigned lds_address(const void *p)
 // address lds_base + 16*l.  lds_base must be wave-uniform.
 __device__ __forceinline__ void async_copy16(const float *base, unsigned voff, unsigned lds_base)
 {
+    // The "s" constraints need values the compiler has in scalar registers; under register pressure
+    // it sometimes computes uniform values on the vector unit, so pin them (a no-op when already scalar).
+    const size_t b = reinterpret_cast<size_t>(base);
+    const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(b));
+    const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(b >> 32));
+    base = reinterpret_cast<const float *>((static_cast<size_t>(hi) << 32) | lo);
+    lds_base = __builtin_amdgcn_readfirstlane(lds_base);
     asm volatile(
         "s_mov_b32 m0, %2\n\t"
         "s_nop 0\n\t"
@@ -390,63 +409,91 @@ __device__ __forceinline__ void wait_vmcnt()
     asm volatile("" ::: "memory");
 }
 
+// Dynamic LDS the async kernel needs at launch: NSTAGE ring slots of one A and one B tile (the B
+// tile padded by 64 bytes per KiB with 16x16 MFMAs).  Above 64 KiB the launcher must first raise
+// hipFuncAttributeMaxDynamicSharedMemorySize.
+template <typename Cfg, int NSTAGE>
+constexpr int async_lds_bytes()
+{
+    constexpr int nbw = Cfg::BK * Cfg::BN / 4 / 64, bpad = Cfg::MF == 16 ? 16 : 0;
+    return NSTAGE * (Cfg::BM * Cfg::BK + Cfg::BK * Cfg::BN + nbw * bpad) * 4;
+}
+
 // BF16: the operands are rounded to bf16 (round-to-nearest-even, v_cvt_pk_bf16_f32) after they are read
 // from LDS and multiplied with v_mfma_f32_32x32x16_bf16; accumulation, fold and stores stay fp32.
 // ABL: timing ablations for kernel development (bit 0: no barrier, 1: no copy wait, 2: no copies,
-// 3: no LDS reads); results are wrong with any bit set.  Always 0 in the library.
+// 3: no LDS reads, 4: no output stores); results are wrong with any bit set.  Always 0 in the library.
 template <typename Cfg, int NSTAGE, bool BF16 = false, int ABL = 0>
 __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_mfma_async_kernel(
     const float *__restrict__ TI, const float *__restrict__ Wt, float *__restrict__ Out, size_t M, int C, int K, int nH,
-    int nW, unsigned tiles_n)
+    int nW, unsigned tiles_n, unsigned rows_per_wg)
 {
-    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
-    constexpr int TM = Cfg::TM, TN = Cfg::TN, NA = Cfg::NA, NB = Cfg::NB;
-    constexpr int KS = BK / 8, CH = BK / 4, NWAVES = NT / 64;
-    constexpr int A_FLOATS = BM * BK, B_FLOATS = BK * BN, STAGE_FLOATS = A_FLOATS + B_FLOATS;
-    constexpr int LPS = NA + NB;  // loads per thread per step
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT, MF = Cfg::MF, LG = Cfg::LG, KG = Cfg::KG;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN;
+    constexpr int KS = BK / KG, CH = BK / 4, NWAVES = NT / 64;
+    // Copies are wave-wide: 64 lanes x 16 bytes = 1 KiB.  NAW / NBW of them make an A / B tile; every
+    // wave issues the same number (NA + NB) per step so that all waves count outstanding copies alike;
+    // where the tile does not divide evenly the surplus copies repeat an earlier one (same bytes twice).
+    constexpr int NAW = BM * CH / 64, NBW = BK * BN / 4 / 64;
+    constexpr int NA = (NAW + NWAVES - 1) / NWAVES, NB = (NBW + NWAVES - 1) / NWAVES;
+    // With 16x16 MFMAs the four lane groups of a B operand read hit rows 4 apart; 64 bytes of padding
+    // after every copy (4 rows of 64 floats) put them on different banks.
+    constexpr int BPAD = MF == 16 ? 16 : 0;  // floats
+    static_assert(BPAD == 0 || BN == 64, "the padded B layout assumes one copy = 4 rows");
+    constexpr int A_FLOATS = BM * BK, B_FLOATS = BK * BN + NBW * BPAD, STAGE_FLOATS = A_FLOATS + B_FLOATS;
+    constexpr int LPS = NA + NB;  // copies per thread per step
     static_assert(NSTAGE >= 2, "a ring needs two slots");
     static_assert(KS % 2 == 0, "the MFMA chain of a step is split in two halves");
-    static_assert(!BF16 || KS == 4, "the bf16 MFMA consumes 16 reduction indices: a half of a 32-index step");
+    static_assert(!BF16 || (KS == 4 && MF == 32), "the bf16 MFMA consumes 16 reduction indices: a half of a 32-index step");
     static_assert((CH & (CH - 1)) == 0, "swizzle needs a power-of-two chunk count");
-    static_assert(BM % (64 / CH) == 0 && (BM * CH) % 64 == 0 && (BK * BN / 4) % 64 == 0, "whole wave-loads");
+    static_assert((BM * CH) % 64 == 0 && (BK * BN / 4) % 64 == 0, "tiles are whole wave-wide copies");
     static_assert((NSTAGE - 2) * LPS < 64, "vmcnt range");
 
-    __shared__ __attribute__((aligned(1024))) float smem[NSTAGE * STAGE_FLOATS];
+    static_assert(NSTAGE * STAGE_FLOATS * 4 == async_lds_bytes<Cfg, NSTAGE>(), "launcher and kernel agree on the LDS size");
+    extern __shared__ __attribute__((aligned(1024))) float smem[];  // async_lds_bytes<Cfg, NSTAGE>() bytes
 
     const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
-    const size_t m0 = static_cast<size_t>(lid / tiles_n) * BM;
+    // The workgroup's tile starts at row m0 and is BM rows tall, of which the first rows_valid are
+    // its own (rows_per_wg <= BM lets the launcher split M evenly at 16-row granularity).
+    const size_t m0 = static_cast<size_t>(lid / tiles_n) * rows_per_wg;
     const int n0 = static_cast<int>(lid % tiles_n) * BN;
-    const unsigned rows_valid = static_cast<unsigned>(M - m0 < BM ? M - m0 : BM);
+    const unsigned rows_valid = static_cast<unsigned>(M - m0 < rows_per_wg ? M - m0 : rows_per_wg);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int li = lane & 31, lg = lane >> 5;
+    const int li = lane % MF, lg = lane / MF;
     const int wm0 = (wave / Cfg::WGN) * Cfg::WM, wn0 = (wave % Cfg::WGN) * Cfg::WN;
 
     // Per-thread byte offsets of the copies (constant over the whole kernel) and the
     // wave-uniform LDS byte offsets, relative to a stage, they land at.
     unsigned a_voff[NA], b_voff[NB];
+    unsigned a_lds[NA], b_lds[NB];  // wave-uniform byte offsets within a stage
+    const unsigned wave_u = __builtin_amdgcn_readfirstlane(wave);
 #pragma unroll
     for (int q = 0; q < NA; ++q) {
-        const unsigned slot = (q * NWAVES + wave) * 64 + lane;
+        const unsigned wl = (q * NWAVES + wave_u) % NAW;
+        const unsigned slot = wl * 64 + lane;
         unsigned row = slot / CH;
         const unsigned chunk = (slot % CH) ^ (row % CH);
         row = row < rows_valid ? row : rows_valid - 1;
         a_voff[q] = (row * static_cast<unsigned>(C) + chunk * 4) * 4u;
+        a_lds[q] = wl * 1024u;
     }
 #pragma unroll
     for (int q = 0; q < NB; ++q) {
-        const unsigned slot = (q * NWAVES + wave) * 64 + lane;
+        const unsigned wl = (q * NWAVES + wave_u) % NBW;
+        const unsigned slot = wl * 64 + lane;
         const unsigned krow = slot / (BN / 4);
         unsigned n = n0 + (slot % (BN / 4)) * 4;
         n = n + 4 <= static_cast<unsigned>(K) ? n : static_cast<unsigned>(K) - 4;
         b_voff[q] = (krow * static_cast<unsigned>(K) + n) * 4u;
+        b_lds[q] = A_FLOATS * 4 + wl * (1024u + BPAD * 4);
     }
     const unsigned smem_base = lds_address(smem);
-    const unsigned wave_lds = __builtin_amdgcn_readfirstlane(wave) * 1024u;
 
     const int nkc = C / BK;
-    floatx16 Y[4][TM][TN];
+    using Acc = AccT<Cfg>;
+    Acc Y[4][TM][TN];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -454,7 +501,7 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) Y[j][tm][tn][r] = 0.f;
+                for (int r = 0; r < Cfg::REGS; ++r) Y[j][tm][tn][r] = 0.f;
 
     // ---- copy issuer: running pointers to the tiles of the next step to fetch -------------
     // Tile of (pos, c0): A at TI + (pos*M + m0)*C + c0, B at Wt + (pos*C + c0)*K.  Consecutive
@@ -464,19 +511,19 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     const size_t a_wrap = (M - 1) * static_cast<size_t>(C);
     const size_t b_inc = static_cast<size_t>(BK) * K;
     int kc_next = 0, pos_next = 0;
-    unsigned lds_next = smem_base + wave_lds;  // this wave's first copy target in the next ring slot
+    unsigned lds_next = smem_base;  // byte address of the next ring slot
     int slot_next = 0;
-    auto copy = [&](int i) {  // the i-th of this thread's LPS copies of a step
+    auto copy = [&](int i) __attribute__((always_inline)) {  // the i-th of this thread's LPS copies of a step
         if (i < NA)
-            async_copy16(a_next, a_voff[i < NA ? i : 0], lds_next + i * (NWAVES * 1024));
+            async_copy16(a_next, a_voff[i < NA ? i : 0], lds_next + a_lds[i < NA ? i : 0]);
         else
-            async_copy16(b_next, b_voff[i >= NA ? i - NA : 0], lds_next + A_FLOATS * 4 + (i - NA) * (NWAVES * 1024));
+            async_copy16(b_next, b_voff[i >= NA ? i - NA : 0], lds_next + b_lds[i >= NA ? i - NA : 0]);
     };
     // After the last step the issuer wraps around to the first tile again: the loop below
     // issues one step's copies per step unconditionally (so the outstanding-copy count is the
     // same at every wait), and the surplus copies at the end re-fetch valid memory into ring
     // slots nobody reads any more.
-    auto advance = [&]() {
+    auto advance = [&]() __attribute__((always_inline)) {
         a_next += BK;
         b_next += b_inc;
         if (++kc_next == nkc) {
@@ -491,15 +538,16 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
         lds_next += STAGE_FLOATS * 4;
         if (++slot_next == NSTAGE) {
             slot_next = 0;
-            lds_next = smem_base + wave_lds;
+            lds_next = smem_base;
         }
     };
 
     // ---- MFMA operands ---------------------------------------------------------------------
-    // A step's reduction range BK is consumed in two halves of KH groups of 8 indices.  Within
-    // a group, lane group lg feeds indices 4*lg .. 4*lg+3, one per MFMA (the order in which
-    // indices are reduced is free as long as A and B agree), so A comes as one b128 read per
-    // group and B as 4 b32 reads, paired so that they merge into ds_read2_b32.
+    // A step's reduction range BK is consumed in two halves of KH groups of KG indices (8 with
+    // 32x32 MFMAs, 16 with 16x16).  Within a group, lane group lg feeds indices 4*lg .. 4*lg+3,
+    // one per MFMA (the order in which indices are reduced is free as long as A and B agree), so
+    // A comes as one b128 read per group and B as 4 b32 reads, paired so that they merge into
+    // ds_read2_b32.
     constexpr int KH = KS / 2;
     struct HalfFrag {
         float4 a[KH][TM];
@@ -515,21 +563,23 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     for (int k8 = 0; k8 < KS; ++k8)
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
-            const int row = wm0 + tm * 32 + li;
-            a_off[k8][tm] = row * CH + ((2 * k8 + lg) ^ (row % CH));  // in 16-byte units
+            const int row = wm0 + tm * MF + li;
+            a_off[k8][tm] = row * CH + ((LG * k8 + lg) ^ (row % CH));  // in 16-byte units
         }
-    const int b_off = A_FLOATS + 4 * lg * BN + wn0 + li;
+    // B row k sits at k*BN floats plus BPAD per 4 rows; lane group lg reads rows 4*lg + t of a group.
+    constexpr int BROW4 = 4 * BN + BPAD;
+    const int b_off = A_FLOATS + lg * BROW4 + wn0 + li;
 
     // Read unit u of half h of the stage at float offset st into F.
-    auto read_unit = [&](HalfFrag &F, int st, int h, int u) {
+    auto read_unit = [&](HalfFrag &F, int st, int h, int u) __attribute__((always_inline)) {
         const int k8l = u / (TM + 2 * TN), v = u % (TM + 2 * TN);
         const int k8 = h * KH + k8l;
         if (v < TM) {
             F.a[k8l][v] = reinterpret_cast<const float4 *>(smem)[st / 4 + a_off[k8][v]];
         } else {
             const int tn = (v - TM) / 2, tp = (v - TM) % 2;
-            F.b[k8l][2 * tp][tn] = smem[st + b_off + (k8 * 8 + 2 * tp) * BN + tn * 32];
-            F.b[k8l][2 * tp + 1][tn] = smem[st + b_off + (k8 * 8 + 2 * tp + 1) * BN + tn * 32];
+            F.b[k8l][2 * tp][tn] = smem[st + b_off + k8 * LG * BROW4 + (2 * tp) * BN + tn * MF];
+            F.b[k8l][2 * tp + 1][tn] = smem[st + b_off + k8 * LG * BROW4 + (2 * tp + 1) * BN + tn * MF];
         }
     };
     // ---- prologue: fill the ring, wait for step 0, read its first half ----------------------
@@ -560,14 +610,14 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     // way over the first step of the next position, which accumulates into the other of two
     // product buffers and starts its chains from a zero accumulator.
     int st_cur = 0;  // float offset of the ring slot of the current step
-    floatx16 P[2][TM][TN];
-    const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    Acc P[2][TM][TN];
+    const Acc zero16 = {};
 
     // Fold unit e of position `pos` (e = j*TM*TN + tm*TN + tn): Y_j +-= P.  The empty asm pins the
     // update here: Y is not read again until the final stores, so without it the compiler defers
     // all the adds to the end and keeps the 16 product tiles alive instead of the 4 sums.
     constexpr int NE = 4 * TM * TN;
-    auto fold_unit = [&](const floatx16 (&Pp)[TM][TN], int pos, int e) {
+    auto fold_unit = [&](const Acc (&Pp)[TM][TN], int pos, int e) __attribute__((always_inline)) {
         constexpr unsigned long long plus = kPlus, minus = kMinus;
         const int j = e / (TM * TN), tm = (e / TN) % TM, tn = e % TN;
         const int bit = 4 * pos + j;
@@ -582,11 +632,11 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
 
     // One step.  first: the chains start from zero and the fold of position fold_pos (held in
     // Pprev) rides along; otherwise fold_pos is ignored.
-    auto step = [&](floatx16 (&Pc)[TM][TN], const floatx16 (&Pprev)[TM][TN], auto first_tag, auto fold_tag) {
+    auto step = [&](Acc (&Pc)[TM][TN], const Acc (&Pprev)[TM][TN], auto first_tag, auto fold_tag) __attribute__((always_inline)) {
         constexpr bool first = decltype(first_tag)::value;
         constexpr int fold_pos = decltype(fold_tag)::value;
         const int st_next = st_cur + STAGE_FLOATS == NSTAGE * STAGE_FLOATS ? 0 : st_cur + STAGE_FLOATS;
-        auto mfma_slot = [&](const HalfFrag &F, int i, bool from_zero) {
+        auto mfma_slot = [&](const HalfFrag &F, int i, bool from_zero) __attribute__((always_inline)) {
             if constexpr (BF16) {
                 // Lane group lg holds reduction indices {8*k8l + 4*lg + t}: 8 per half, the same
                 // set on the A and the B side, which is all the MFMA needs.
@@ -603,7 +653,10 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
                 const int tn = i % TN, tm = (i / TN) % TM, t = (i / (TN * TM)) % 4, k8l = i / (TN * TM * 4);
                 const float4 a4 = F.a[k8l][tm];
                 const float av = t == 0 ? a4.x : t == 1 ? a4.y : t == 2 ? a4.z : a4.w;
-                Pc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, F.b[k8l][t][tn], from_zero ? zero16 : Pc[tm][tn], 0, 0, 0);
+                if constexpr (MF == 32)
+                    Pc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, F.b[k8l][t][tn], from_zero ? zero16 : Pc[tm][tn], 0, 0, 0);
+                else
+                    Pc[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, F.b[k8l][t][tn], from_zero ? zero16 : Pc[tm][tn], 0, 0, 0);
             }
         };
         // Slots (MFMA indices of the second half) after which the copies and LDS reads go; all
@@ -665,7 +718,7 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     // The surplus copies must have landed before this workgroup's LDS can be handed on.
     wait_vmcnt<0>();
 
-    store_output<Cfg>(Y, Out, M, K, nW, m0, n0, wm0, wn0, li, lg);
+    if (!(ABL & 16) || nH < 0) store_output<Cfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg);
 }
 
 }  // namespace

@@ -238,7 +238,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
     });
     using StoreCfg = ConvCfg<FBM, FBN, 32, 2, 2>;
-    store_output<StoreCfg>(Y, Out, M, K, nW, m0, n0, wm0, wn0, li, lg);
+    const unsigned rows_valid = static_cast<unsigned>(M - m0 < FBM ? M - m0 : FBM);
+    store_output<StoreCfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg);
 }
 
 }  // namespace

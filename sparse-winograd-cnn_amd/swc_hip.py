@@ -20,7 +20,7 @@ SWC_ERR_UNSUPPORTED = -6
 
 # Every symbol include/winograd2x2.h declares with C linkage.
 C_SYMBOLS = (
-    "swc_strerror", "swc_last_hip_error", "swc_version",
+    "swc_strerror", "swc_last_hip_error", "swc_version", "swc_winograd2x2_conv_last_kernel",
     "swc_winograd2x2_imtrans", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
@@ -68,6 +68,8 @@ def lib():
         L.swc_last_hip_error.argtypes = []
         L.swc_version.restype = ctypes.c_char_p
         L.swc_version.argtypes = []
+        L.swc_winograd2x2_conv_last_kernel.restype = ctypes.c_char_p
+        L.swc_winograd2x2_conv_last_kernel.argtypes = []
         L.swc_winograd2x2_imtrans.restype = i32
         L.swc_winograd2x2_imtrans.argtypes = [fp, fp] + [i32] * 7 + [vp]
         for f in (L.swc_winograd2x2_conv, L.swc_winograd2x2_conv_bf16):

@@ -103,6 +103,9 @@ CONV_SHAPES = [
     (2, 3, 3, 96, 132),    # K = 2 tiles + 4 columns
     (1, 1, 1, 32, 4),      # one tile row, one column group
     (5, 9, 11, 160, 72),   # M = 495 (ragged last tile), C = 5 steps
+    (8, 9, 9, 128, 72),    # short row groups (16x16 MFMAs), ragged rows and columns
+    (63, 14, 14, 128, 120),  # tall row groups of 97 rows, last one 29; K = 2 tiles - 8 columns
+    (32, 28, 28, 64, 64),  # tall row groups, one 64-channel reduction in two steps
 ]
 
 
@@ -130,7 +133,20 @@ def test_conv_fp32_matches_oracle(oracle, dev, shape):
     assert rel_l1(got, want) <= TOL
 
 
-@pytest.mark.parametrize("shape", [(3, 3, 3, 32, 32), (2, 4, 4, 5, 7), (2, 3, 5, 36, 100)])
+def test_conv_shapes_reach_every_kernel(dev):
+    # The launcher picks a kernel from the shapes alone; the parity shapes above must cover all five.
+    import swc_hip
+    _, conv = ops()
+    seen = set()
+    for shape in CONV_SHAPES:
+        B, nH, nW, C, K = shape
+        conv(torch.zeros((16, B, nH, nW, C), device=dev), torch.zeros((16, C, K), device=dev))
+        seen.add(swc_hip.lib().swc_winograd2x2_conv_last_kernel().decode())
+    assert seen == {"sync", "ring32", "ring16", "tall16", "short16"}, seen
+
+
+@pytest.mark.parametrize("shape", [(3, 3, 3, 32, 32), (2, 4, 4, 5, 7), (2, 3, 5, 36, 100), (8, 9, 9, 128, 72),
+                                   (63, 14, 14, 128, 120)])
 def test_conv_fp32_exact_on_integers(oracle, dev, shape):
     # Small integers make every product and partial sum exact in fp32, whatever the
     # reduction order: the kernel must equal the oracle bit for bit, which pins operand
