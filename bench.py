@@ -29,7 +29,7 @@ for _p in (ROOT, PKG):
 # HBM traffic per launch (bytes), measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
 # what the same counters read for a 128 MiB copy (profiles/*_pmc_traffic.md); None where not measured.
 MEASURED_TRAFFIC = {
-    ("cfg3", "fp32", "conv"): 148.0e6,     # 122.3 MB fetched + 25.69 MB written (algorithmic 129.5 MB)
+    ("cfg3", "fp32", "conv"): 141.0e6,     # 115.3 MB fetched + 25.69 MB written (algorithmic 129.5 MB)
     ("cfg3", "fp32", "imtrans"): 131.9e6,  # 29.2 MB fetched + 102.76 MB written (algorithmic 128.45 MB)
 }
 

@@ -422,7 +422,7 @@ constexpr int async_lds_bytes()
 // BF16: the operands are rounded to bf16 (round-to-nearest-even, v_cvt_pk_bf16_f32) after they are read
 // from LDS and multiplied with v_mfma_f32_32x32x16_bf16; accumulation, fold and stores stay fp32.
 // ABL: timing ablations for kernel development (bit 0: no barrier, 1: no copy wait, 2: no copies,
-// 3: no LDS reads, 4: no output stores); results are wrong with any bit set.  Always 0 in the library.
+// 3: no LDS reads, 4: no output stores, 5: fold only the last position); results are wrong with any bit set.  Always 0 in the library.
 template <typename Cfg, int NSTAGE, bool BF16 = false, int ABL = 0>
 __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_mfma_async_kernel(
     const float *__restrict__ TI, const float *__restrict__ Wt, float *__restrict__ Out, size_t M, int C, int K, int nH,
@@ -621,7 +621,9 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
         constexpr unsigned long long plus = kPlus, minus = kMinus;
         const int j = e / (TM * TN), tm = (e / TN) % TM, tn = e % TN;
         const int bit = 4 * pos + j;
-        if ((plus >> bit) & 1ull) {
+        if (ABL & 32) {
+            if (pos == 15) Y[j][tm][tn] += Pp[tm][tn];
+        } else if ((plus >> bit) & 1ull) {
             Y[j][tm][tn] += Pp[tm][tn];
             asm volatile("" : "+v"(Y[j][tm][tn]));
         } else if ((minus >> bit) & 1ull) {
