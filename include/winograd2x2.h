@@ -67,6 +67,20 @@ SWC_API int swc_winograd2x2_imtrans(const float *Input, float *TransIm, int C, i
                             int pad_h, int pad_w, int relu, swc_stream_t stream);
 
 /*
+ * swc_winograd2x2_imtrans with a per-channel affine map folded into the load: every pixel inside
+ * the image becomes fmaf(x, Scale[c], Shift[c]) before the transform; the zero padding stays zero.
+ *   Scale, Shift [C] fp32
+ * This is the inference-mode BatchNorm that precedes every WinogradImTrans in the reference model
+ * (`BatchNorm('bn2a_2a', x)` then `WinogradImTrans(..., tf.nn.relu)`,
+ * ResNet-18-var/imagenet-resnet-transWino-prune.py:117-118 and the 15 other pairs up to :210), with
+ * Scale = gamma / sqrt(var + eps), Shift = beta - mean * Scale: one pass over the activations
+ * instead of two.  The reference has no single function for the pair.
+ */
+SWC_API int swc_winograd2x2_imtrans_affine(const float *Input, const float *Scale, const float *Shift,
+                                   float *TransIm, int C, int B, int H, int W, int pad_h, int pad_w, int relu,
+                                   swc_stream_t stream);
+
+/*
  * The 16 per-position products TI[i] (MxC) . Weight[i] (CxK), M = B*nH*nW, followed by
  * the output transform Y = A^T p A, in one kernel (fp32 MFMA, fp32 accumulate).
  *   Input  [16,B,nH,nW,C]  fp32      Weight [16,C,K] fp32

@@ -72,6 +72,26 @@ def imtrans(x, relu=False):
     return out
 
 
+def affine(x, scale, shift):
+    """x [...,C] -> fmaf(x, scale[c], shift[c]) elementwise, fp32 with a single rounding."""
+    x, xp = _f32(x)
+    scale, sp = _f32(scale)
+    shift, hp = _f32(shift)
+    C = x.shape[-1]
+    assert scale.shape == (C,) and shift.shape == (C,)
+    out = np.empty_like(x)
+    L = lib()
+    L.oracle_affine_f32.argtypes = [_F, _F, _F, _F, ctypes.c_long, ctypes.c_int]
+    L.oracle_affine_f32.restype = None
+    L.oracle_affine_f32(xp, sp, hp, out.ctypes.data_as(_F), x.size // C, C)
+    return out
+
+
+def imtrans_affine(x, scale, shift, relu=False):
+    """Transform of the affinely mapped image (zero padding stays zero): imtrans(affine(x))."""
+    return imtrans(affine(x, scale, shift), relu=relu)
+
+
 def gemm16(ti, w, acc64=False):
     """ti [16,M,C] (any leading tile dims), w [16,C,K] -> P [16,M,K] fp32."""
     ti, tp = _f32(ti)

@@ -23,12 +23,15 @@
  *   oracle_gemm16_*           numpy float64 matmul
  *   oracle_output_transform   matrix form A^T p A in float64 numpy
  *   oracle_kernel_transform   matrix form G g G^T in float64 numpy
+ *   oracle_affine_f32         float64 x*s+t on inputs where that sum is exact, so that rounding
+ *                             it once to fp32 is the fused result (and differs from mul-then-add)
  *   whole path (nl=identity)  conv2d(x, g, stride 1, pad 1) from torch on the CPU,
  *                             the same relation the reference's own tests print
  *                             (CVT:177,187-204), plus a direct 3x3 loop nest
  *   The summation order inside cuBLAS is unspecified, so bitwise parity of the
  *   GEMM stage is unpinned by construction; it is held to a tolerance instead.
  */
+#include <math.h>
 #include <stddef.h>
 #include <stdint.h>
 #include <string.h>
@@ -315,6 +318,21 @@ ORACLE_API void oracle_conv_grad_f32(const float *TI, const float *Wt, const flo
             for (int k = 0; k < K; ++k) dW[((size_t)i * C + c) * K + k] = (float)acc[k];
         }
 }
+
+/*
+ * Per-channel affine map ahead of the transform: y = fmaf(x, scale[c], shift[c]) on every pixel of
+ * X [B,H,W,C] (the padding the transform adds afterwards stays zero).  Restates the reference
+ * model's BatchNorm-then-WinogradImTrans pairs at inference
+ * (ResNet-18-var/imagenet-resnet-transWino-prune.py:117-118 ... :209-210) with the normalisation
+ * reduced to scale = gamma/sqrt(var+eps), shift = beta - mean*scale.  fmaf rounds once.
+ */
+ORACLE_API void oracle_affine_f32(const float *X, const float *scale, const float *shift, float *Y, long pixels, int C)
+{
+#pragma omp parallel for schedule(static)
+    for (long p = 0; p < pixels; ++p)
+        for (int c = 0; c < C; ++c) Y[p * C + c] = fmaf(X[p * C + c], scale[c], shift[c]);
+}
+
 
 /*
  * Winograd2x2ImTransGrad: dX = sum over tiles of (B dT B^T) scattered back onto the 4x4 patch the

@@ -442,6 +442,8 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     static_assert(BPAD == 0 || BN == 64, "the padded B layout assumes one copy = 4 rows");
     constexpr int A_FLOATS = BM * BK, B_FLOATS = BK * BN + NBW * BPAD, STAGE_FLOATS = A_FLOATS + B_FLOATS;
     constexpr int LPS = NA + NB;  // copies per thread per step
+    // Scheduling granularity (development knobs): reads/copies are dealt out in groups of GR, fold units in groups of GF.
+    constexpr int GR = ((ABL >> 8) & 15) ? ((ABL >> 8) & 15) : 1, GF = ((ABL >> 12) & 31) ? ((ABL >> 12) & 31) : 1;
     static_assert(NSTAGE >= 2, "a ring needs two slots");
     static_assert(KS % 2 == 0, "the MFMA chain of a step is split in two halves");
     static_assert(!BF16 || (KS == 4 && MF == 32), "the bf16 MFMA consumes 16 reduction indices: a half of a 32-index step");
@@ -663,18 +665,18 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
         };
         // Slots (MFMA indices of the second half) after which the copies and LDS reads go; all
         // behind the barrier that follows MFMA 0.
-        auto copy_slot = [](int c) { return NM > 1 ? 1 + c * (NM - 1) / LPS : 0; };
-        auto read_slot = [](int u) { return NM > 1 ? 1 + u * (NM - 1) / NU : 0; };
+        auto copy_slot = [](int c) { return NM > 1 ? 1 + (c / GR * GR) * (NM - 1) / LPS : 0; };
+        auto read_slot = [](int u) { return NM > 1 ? 1 + (u / GR * GR) * (NM - 1) / NU : 0; };
 #pragma unroll
         for (int i = 0; i < NM; ++i) {
             mfma_slot(F1, i, first && i < TM * TN);
 #pragma unroll
             for (int u = 0; u < NU; ++u)
-                if (u * NM / NU == i && !(ABL & 8)) read_unit(F2, st_cur, 1, u);
+                if ((u / GR * GR) * NM / NU == i && !(ABL & 8)) read_unit(F2, st_cur, 1, u);
             if (first && fold_pos >= 0) {
 #pragma unroll
                 for (int e = 0; e < NE; ++e)
-                    if (e * (2 * NM) / NE == i) fold_unit(Pprev, fold_pos, e);
+                    if ((e / GF * GF) * (2 * NM) / NE == i) fold_unit(Pprev, fold_pos, e);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -698,7 +700,7 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
             if (first && fold_pos >= 0) {
 #pragma unroll
                 for (int e = 0; e < NE; ++e)
-                    if (e * (2 * NM) / NE == NM + i) fold_unit(Pprev, fold_pos, e);
+                    if ((e / GF * GF) * (2 * NM) / NE == NM + i) fold_unit(Pprev, fold_pos, e);
             }
             __builtin_amdgcn_sched_barrier(0);
         }

@@ -84,10 +84,15 @@ __device__ __forceinline__ void transform_vec(const typename Vec<VEC>::type (&d)
 // [M, C/VEC] plane of the output, so each of the 16 stores of a wavefront covers
 // 64*VEC*4 contiguous bytes of one plane whatever C is; the 16 loads of a wavefront
 // are contiguous per tile and overlap between neighbouring tiles in L1/L2.
-template <int VEC, bool RELU, typename Idx>
+//
+// AFFINE: every pixel inside the image is first mapped to fma(x, scale[c], shift[c]) (an inference-mode
+// batch normalisation folded into the load); the zero padding stays zero, as it does when the
+// normalisation runs as its own pass before the transform.
+template <int VEC, bool RELU, bool AFFINE, typename Idx>
 __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__restrict__ X, float *__restrict__ TI,
-                                                             int H, int W, int C, int nH, int nW, Idx items,
-                                                             size_t plane)
+                                                             const float *__restrict__ scale,
+                                                             const float *__restrict__ shift, int H, int W, int C,
+                                                             int nH, int nW, Idx items, size_t plane)
 {
     using V = typename Vec<VEC>::type;
     // Consecutive logical blocks share input rows (the halo between tile rows, the overlap
@@ -106,6 +111,11 @@ __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__rest
     const int y0 = 2 * th - 1, x0 = 2 * tw - 1;
     const float *img = X + b * H * W * C + static_cast<size_t>(cv) * VEC;
     V d[16];
+    V sc = Vec<VEC>::zero(), sh = Vec<VEC>::zero();
+    if (AFFINE) {
+        sc = *reinterpret_cast<const V *>(scale + static_cast<size_t>(cv) * VEC);
+        sh = *reinterpret_cast<const V *>(shift + static_cast<size_t>(cv) * VEC);
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int y = y0 + r;
@@ -114,8 +124,16 @@ __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__rest
         for (int s = 0; s < 4; ++s) {
             const int x = x0 + s;
             const bool in = yin && (x > -1) && (x < W);
-            d[4 * r + s] = in ? *reinterpret_cast<const V *>(img + (static_cast<size_t>(y) * W + x) * C)
-                              : Vec<VEC>::zero();
+            V v = Vec<VEC>::zero();
+            if (in) {
+                v = *reinterpret_cast<const V *>(img + (static_cast<size_t>(y) * W + x) * C);
+                if (AFFINE) {
+#pragma unroll
+                    for (int q = 0; q < VEC; ++q)
+                        Vec<VEC>::set(v, q, __builtin_fmaf(Vec<VEC>::get(v, q), Vec<VEC>::get(sc, q), Vec<VEC>::get(sh, q)));
+                }
+            }
+            d[4 * r + s] = v;
         }
     }
     V t[16];
@@ -125,15 +143,40 @@ __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__rest
     for (int i = 0; i < 16; ++i) *reinterpret_cast<V *>(dst + i * plane) = t[i];
 }
 
-template <int VEC, bool RELU, typename Idx>
-int launch_direct(const float *X, float *TI, int B, int H, int W, int C, int nH, int nW, hipStream_t stream)
+template <int VEC, bool RELU, bool AFFINE, typename Idx>
+int launch_direct(const float *X, const float *scale, const float *shift, float *TI, int B, int H, int W, int C, int nH,
+                  int nW, hipStream_t stream)
 {
     const size_t M = static_cast<size_t>(B) * nH * nW;
     const size_t items = M * (C / VEC);
     const size_t blocks = (items + 255) / 256;
-    imtrans_direct_kernel<VEC, RELU, Idx><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(
-        X, TI, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
+    imtrans_direct_kernel<VEC, RELU, AFFINE, Idx><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(
+        X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
     return check_launch();
+}
+
+template <bool AFFINE>
+int imtrans_entry(const float *Input, const float *Scale, const float *Shift, float *TransIm, int C, int B, int H, int W,
+                  int pad_h, int pad_w, int relu, swc_stream_t stream)
+{
+    if (Input == nullptr || TransIm == nullptr) return SWC_ERR_NULL_POINTER;
+    if (AFFINE && (Scale == nullptr || Shift == nullptr)) return SWC_ERR_NULL_POINTER;
+    if (C <= 0 || B <= 0 || H <= 0 || W <= 0) return SWC_ERR_BAD_DIMS;
+    if (pad_h != 1 || pad_w != 1) return SWC_ERR_BAD_PAD;
+    const int nH = (H + 1) / 2, nW = (W + 1) / 2;
+    const size_t M = static_cast<size_t>(B) * nH * nW;
+    // One lane per item, 256 per workgroup, grid.x below 2^31.
+    if (M * C / 256 >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool vec = (C % 4 == 0) && aligned16(Input) && aligned16(TransIm) &&
+                     (!AFFINE || (aligned16(Scale) && aligned16(Shift)));
+    const bool small = M * C < (1ull << 31);
+#define SWC_DISPATCH(VEC, RELU)                                                                                    \
+    (small ? launch_direct<VEC, RELU, AFFINE, unsigned>(Input, Scale, Shift, TransIm, B, H, W, C, nH, nW, s)       \
+           : launch_direct<VEC, RELU, AFFINE, unsigned long long>(Input, Scale, Shift, TransIm, B, H, W, C, nH, nW, s))
+    if (vec) return relu ? SWC_DISPATCH(4, true) : SWC_DISPATCH(4, false);
+    return relu ? SWC_DISPATCH(1, true) : SWC_DISPATCH(1, false);
+#undef SWC_DISPATCH
 }
 
 }  // namespace
@@ -142,21 +185,12 @@ int launch_direct(const float *X, float *TI, int B, int H, int W, int C, int nH,
 extern "C" int swc_winograd2x2_imtrans(const float *Input, float *TransIm, int C, int B, int H, int W,
                                        int pad_h, int pad_w, int relu, swc_stream_t stream)
 {
-    using namespace swc;
-    if (Input == nullptr || TransIm == nullptr) return SWC_ERR_NULL_POINTER;
-    if (C <= 0 || B <= 0 || H <= 0 || W <= 0) return SWC_ERR_BAD_DIMS;
-    if (pad_h != 1 || pad_w != 1) return SWC_ERR_BAD_PAD;
-    const int nH = (H + 1) / 2, nW = (W + 1) / 2;
-    const size_t M = static_cast<size_t>(B) * nH * nW;
-    // One lane per item, 256 per workgroup, grid.x below 2^31.
-    if (M * C / 256 >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool vec = (C % 4 == 0) && aligned16(Input) && aligned16(TransIm);
-    const bool small = M * C < (1ull << 31);
-#define SWC_DISPATCH(VEC, RELU)                                                           \
-    (small ? launch_direct<VEC, RELU, unsigned>(Input, TransIm, B, H, W, C, nH, nW, s)    \
-           : launch_direct<VEC, RELU, unsigned long long>(Input, TransIm, B, H, W, C, nH, nW, s))
-    if (vec) return relu ? SWC_DISPATCH(4, true) : SWC_DISPATCH(4, false);
-    return relu ? SWC_DISPATCH(1, true) : SWC_DISPATCH(1, false);
-#undef SWC_DISPATCH
+    return swc::imtrans_entry<false>(Input, nullptr, nullptr, TransIm, C, B, H, W, pad_h, pad_w, relu, stream);
+}
+
+extern "C" int swc_winograd2x2_imtrans_affine(const float *Input, const float *Scale, const float *Shift,
+                                              float *TransIm, int C, int B, int H, int W, int pad_h, int pad_w,
+                                              int relu, swc_stream_t stream)
+{
+    return swc::imtrans_entry<true>(Input, Scale, Shift, TransIm, C, B, H, W, pad_h, pad_w, relu, stream);
 }

@@ -11,7 +11,9 @@ stage 5 also runs at 14x14; ReLU, global average pool, (dropout: identity at inf
 after, not before).
 
 Everything except the two Winograd ops is stock PyTorch.  Activations are kept NHWC in memory
-(channels_last), so handing them to the ops and back costs no copies.
+(channels_last), so handing them to the ops and back costs no copies.  The BatchNorm in front of
+each WinogradImTrans (inference statistics) is folded into the transform kernel as a per-channel
+scale and shift; ``fold_bn=False`` runs it as its own pass instead.
 """
 import os
 import sys
@@ -46,6 +48,18 @@ def _same_pad(x, k, stride):
     return pads
 
 
+def _bn_affine(bn):
+    """Inference-mode BatchNorm2d as y = x*scale + shift; cached until a parameter or statistic changes."""
+    tensors = (bn.weight, bn.bias, bn.running_mean, bn.running_var)
+    key = tuple((t._version, t.data_ptr()) for t in tensors)
+    cached = getattr(bn, "_swc_affine", None)
+    if cached is None or cached[0] != key:
+        scale = (bn.weight * torch.rsqrt(bn.running_var + bn.eps)).detach()
+        cached = (key, scale.contiguous(), (bn.bias - bn.running_mean * scale).detach().contiguous())
+        bn._swc_affine = cached
+    return cached[1], cached[2]
+
+
 def _to_nhwc(x):   # NCHW tensor in channels_last memory -> contiguous [B,H,W,C] view
     return x.permute(0, 2, 3, 1).contiguous()
 
@@ -55,9 +69,9 @@ def _to_nchw(y):   # contiguous [B,H,W,C] -> NCHW tensor in channels_last memory
 
 
 class WinogradUnit(torch.nn.Module):
-    def __init__(self, name, c_in, c_out, shortcut, pool, masks, precision):
+    def __init__(self, name, c_in, c_out, shortcut, pool, masks, precision, fold_bn=True):
         super().__init__()
-        self.name, self.pool = name, pool
+        self.name, self.pool, self.fold_bn = name, pool, fold_bn
         self.bn2a = torch.nn.BatchNorm2d(c_in)
         self.conv2a = WinogradConv(c_in, c_out, mask=masks.get("Winograd_W%s_2a/W" % name), precision=precision)
         self.bn2b = torch.nn.BatchNorm2d(c_out)
@@ -70,6 +84,10 @@ class WinogradUnit(torch.nn.Module):
             self.bn1 = torch.nn.BatchNorm2d(c_out)
 
     def branch(self, x):
+        if self.fold_bn:
+            h = self.conv2a(WinogradImTrans(_to_nhwc(x), torch.relu, affine=_bn_affine(self.bn2a)))
+            h = self.conv2b(WinogradImTrans(h, torch.relu, affine=_bn_affine(self.bn2b)))
+            return self.bn2c(_to_nchw(h))
         h = _to_nchw(self.conv2a(WinogradImTrans(_to_nhwc(self.bn2a(x)), torch.relu)))
         h = _to_nchw(self.conv2b(WinogradImTrans(_to_nhwc(self.bn2b(h)), torch.relu)))
         return self.bn2c(h)
@@ -91,12 +109,12 @@ class ResNet18Var(torch.nn.Module):
     """``masks``: optional dict of 0/1 arrays keyed like the reference's pruning masks
     ('Winograd_W2a_2a/W', ...; prune_script.py:68-78).  ``precision``: 'fp32' or 'bf16' GEMM operands."""
 
-    def __init__(self, masks=None, precision="fp32", num_classes=1000):
+    def __init__(self, masks=None, precision="fp32", num_classes=1000, fold_bn=True):
         super().__init__()
         masks = masks or {}
         self.conv1 = torch.nn.Conv2d(3, 64, 7, stride=2, bias=False)
         self.units = torch.nn.ModuleList(
-            [WinogradUnit(n, ci, co, sc, pool, masks, precision) for n, ci, co, sc, pool in UNITS])
+            [WinogradUnit(n, ci, co, sc, pool, masks, precision, fold_bn) for n, ci, co, sc, pool in UNITS])
         self.linear = torch.nn.Linear(512, num_classes)
         self.eval()
 

@@ -21,7 +21,7 @@ SWC_ERR_UNSUPPORTED = -6
 # Every symbol include/winograd2x2.h declares with C linkage.
 C_SYMBOLS = (
     "swc_strerror", "swc_last_hip_error", "swc_version", "swc_winograd2x2_conv_last_kernel",
-    "swc_winograd2x2_imtrans", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
+    "swc_winograd2x2_imtrans", "swc_winograd2x2_imtrans_affine", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
     "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad", "swc_winograd2x2_relu_conv",
@@ -72,6 +72,8 @@ def lib():
         L.swc_winograd2x2_conv_last_kernel.argtypes = []
         L.swc_winograd2x2_imtrans.restype = i32
         L.swc_winograd2x2_imtrans.argtypes = [fp, fp] + [i32] * 7 + [vp]
+        L.swc_winograd2x2_imtrans_affine.restype = i32
+        L.swc_winograd2x2_imtrans_affine.argtypes = [fp, fp, fp, fp] + [i32] * 7 + [vp]
         for f in (L.swc_winograd2x2_conv, L.swc_winograd2x2_conv_bf16):
             f.restype = i32
             f.argtypes = [fp, fp, fp, fp, vp] + [i32] * 7 + [vp]

@@ -22,9 +22,16 @@ def winograd2x2_imTrans_shape(shape):
     return tuple(out)
 
 
-def _forward(I, relu, out):
+def _forward(I, relu, out, scale=None, shift=None):
     I = swc_hip.require_cuda_f32(I, "I", 4)
     shape = winograd2x2_imTrans_shape(I.shape)
+    if (scale is None) != (shift is None):
+        raise ValueError("scale and shift go together")
+    if scale is not None:
+        scale = swc_hip.require_cuda_f32(scale, "scale", 1)
+        shift = swc_hip.require_cuda_f32(shift, "shift", 1)
+        if scale.shape[0] != I.shape[3] or shift.shape[0] != I.shape[3]:
+            raise ValueError("scale and shift must have one entry per channel (%d)" % I.shape[3])
     if out is None:
         out = torch.empty(shape, dtype=torch.float32, device=I.device)
     else:
@@ -32,8 +39,15 @@ def _forward(I, relu, out):
             raise ValueError("out must be a contiguous float32 tensor of shape %s on %s" % (shape, I.device))
     with torch.cuda.device(I.device):
         stream = torch.cuda.current_stream().cuda_stream
-        st = swc_hip.lib().swc_winograd2x2_imtrans_op_compute(
-            I.data_ptr(), 4, swc_hip.dims(I.shape), out.data_ptr(), 5, swc_hip.dims(out.shape), int(bool(relu)), stream)
+        if scale is not None:
+            B, H, W, C = I.shape
+            st = swc_hip.lib().swc_winograd2x2_imtrans_affine(
+                I.data_ptr(), scale.data_ptr(), shift.data_ptr(), out.data_ptr(), C, B, H, W, 1, 1, int(bool(relu)),
+                stream)
+        else:
+            st = swc_hip.lib().swc_winograd2x2_imtrans_op_compute(
+                I.data_ptr(), 4, swc_hip.dims(I.shape), out.data_ptr(), 5, swc_hip.dims(out.shape), int(bool(relu)),
+                stream)
     swc_hip.check(st, "winograd2x2_imTrans")
     return out
 
@@ -85,14 +99,20 @@ class _ImTransFunction(torch.autograd.Function):
         return winograd2x2_imTrans_grad(grad.contiguous(), ctx.hw[0], ctx.hw[1], relu_output), None
 
 
-def winograd2x2_imTrans(I, relu=False, out=None):
+def winograd2x2_imTrans(I, relu=False, out=None, scale=None, shift=None):
     """I: [B,H,W,C] float32 NHWC on the GPU -> [16,B,nH,nW,C].
+
+    ``scale``/``shift`` ([C] each, forward only): the transform of ``I*scale + shift`` (one fused
+    multiply-add per pixel, zero padding left at zero) -- an inference-mode BatchNorm folded into the load.
 
     ``relu=True`` applies the Winograd-domain ReLU inside the same kernel (what
     ``nl(winograd2x2_imTrans(x))`` with ``nl=tf.nn.relu`` computes in
     ResNet-18-var/winograd_imtrans.py:16-17).  ``out`` may supply the result tensor (forward only).
     Differentiable: gradients flow through ``winograd2x2_imTrans_grad``.
     """
-    if out is None and isinstance(I, torch.Tensor) and I.requires_grad and torch.is_grad_enabled():
+    needs_grad = isinstance(I, torch.Tensor) and I.requires_grad and torch.is_grad_enabled()
+    if scale is not None and needs_grad:
+        raise NotImplementedError("the scale/shift variant is forward only")
+    if out is None and needs_grad:
         return _ImTransFunction.apply(I, relu)
-    return _forward(I, relu, out)
+    return _forward(I, relu, out, scale, shift)

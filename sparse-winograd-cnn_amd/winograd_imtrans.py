@@ -17,14 +17,21 @@ def identity(x):
 _RELUS = (torch.relu, torch.nn.functional.relu)
 
 
-def WinogradImTrans(x, nl=identity):
+def WinogradImTrans(x, nl=identity, affine=None):
     """``nl(winograd2x2_imTrans(x))`` as in the reference (winograd_imtrans.py:16-17).
+
+    ``affine=(scale, shift)`` (forward only) transforms ``x*scale + shift`` instead of ``x``: the
+    inference-mode BatchNorm that precedes every call in the reference model, folded into the kernel.
 
     ``nl`` may be a callable or the strings "identity"/"relu".  A ReLU (``torch.relu``,
     ``torch.nn.functional.relu``, an ``nn.ReLU`` module, or "relu") is fused into the
     transform kernel; any other callable is applied to the op's result.
     """
     op = winograd2x2_imTrans.winograd2x2_imTrans.winograd2x2_imTrans
+    if affine is not None:
+        scale, shift = affine
+        base = op
+        op = lambda t, relu=False: base(t, relu=relu, scale=scale, shift=shift)  # noqa: E731
     if nl is None or nl is identity or nl == "identity":
         return op(x)
     if nl == "relu" or isinstance(nl, torch.nn.ReLU) or any(nl is f for f in _RELUS):

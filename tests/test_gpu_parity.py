@@ -332,3 +332,22 @@ def test_layer_wrappers_on_gpu(oracle, dev):
                           torch.tanh(gpu(oracle.imtrans(x), dev)).cpu().numpy())
     y = layer(WinogradImTrans(xd, torch.relu)).detach().cpu().numpy()
     assert rel_max(y, oracle.conv(oracle.imtrans(x, relu=True), w * mask, acc64=True)) <= TOL
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("shape", [(3, 6, 6, 32), (2, 7, 7, 5), (2, 5, 9, 3), (4, 28, 28, 128)])
+def test_imtrans_affine_bit_exact(oracle, dev, shape, relu):
+    # Folded inference BatchNorm: fmaf(x, scale, shift) inside the image, zeros outside, then the transform.
+    imtrans, _ = ops()
+    rng = np.random.default_rng(hash(shape) % 2 ** 31 + 1)
+    x = rng.standard_normal(shape).astype(np.float32)
+    scale = (0.5 + rng.random(shape[3])).astype(np.float32) * rng.choice([-1, 1], shape[3]).astype(np.float32)
+    shift = rng.standard_normal(shape[3]).astype(np.float32)
+    want = oracle.imtrans_affine(x, scale, shift, relu=relu)
+    got = imtrans(gpu(x, dev), relu=relu, scale=gpu(scale, dev), shift=gpu(shift, dev)).cpu().numpy()
+    assert np.array_equal(got == 0, want == 0), "zero mask differs"
+    assert np.array_equal(got, want)
+    # a non-zero shift must not leak into the padding: border tiles differ from transforming a padded-then-mapped image
+    same = imtrans(gpu(oracle.affine(x, scale, shift), dev), relu=relu).cpu().numpy()
+    assert np.array_equal(got, same)

@@ -194,3 +194,23 @@ def test_gen_prune_mask_keeps_largest(oracle):
     assert np.abs(w0[mask == 1]).min() >= np.abs(w0[mask == 0]).max()
     w1 = w0.copy()
     assert oracle.gen_prune_mask(w1, 0.0).all() and np.array_equal(w1, w0)  # rank[:-0] is empty: nothing pruned
+
+
+def test_affine_is_a_single_rounding_fma(oracle):
+    # x, s in [1,2) with full 24-bit significands make 48-bit products; t in [1,4) aligns within
+    # two bits, so x*s+t is exact in float64 and rounding it once to fp32 is the fused result.
+    rng = np.random.default_rng(77)
+    C = 64
+    x = (1 + rng.random((4, 5, 6, C))).astype(np.float32)
+    s = (1 + rng.random(C)).astype(np.float32)
+    t = (1 + 3 * rng.random(C)).astype(np.float32)
+    exact = x.astype(np.float64) * s.astype(np.float64) + t.astype(np.float64)
+    want = exact.astype(np.float32)
+    got = oracle.affine(x, s, t)
+    assert np.array_equal(got, want)
+    # the check has teeth: multiply-then-add rounds twice and differs somewhere
+    assert not np.array_equal((x * s).astype(np.float32) + t, want)
+    # negative scale, zero shift, and the transform of the mapped image
+    s2, t2 = -s, np.zeros_like(t)
+    assert np.array_equal(oracle.affine(x, s2, t2), (-(x.astype(np.float64) * s)).astype(np.float32))
+    assert np.array_equal(oracle.imtrans_affine(x, s, t, relu=True), oracle.imtrans(want, relu=True))

@@ -49,8 +49,11 @@ def test_forward_matches_oracle_path(oracle, precision, tol):
         bn.bias.data.normal_(0, 0.1)
     image = torch.from_numpy(rng.standard_normal((2, 64, 64, 3)).astype(np.float32))
 
-    def cpu_imtrans(x, nl=None):
-        return torch.from_numpy(oracle.imtrans(x.numpy(), relu=True))
+    def cpu_imtrans(x, nl=None, affine=None):
+        x = x.numpy()
+        if affine is not None:
+            x = oracle.affine(x, affine[0].detach().numpy(), affine[1].detach().numpy())
+        return torch.from_numpy(oracle.imtrans(x, relu=True))
 
     def cpu_conv_forward(self, x):
         return torch.from_numpy(oracle.conv(x.numpy(), self.masked_weight().numpy(), acc64=True))
@@ -71,3 +74,11 @@ def test_forward_matches_oracle_path(oracle, precision, tol):
     assert got.shape == want.shape == (2, 1000)
     assert np.isfinite(got).all()
     assert rel_max(got, want) <= tol
+    # Folding the BatchNorm into the transform changes roundings only (one fma per pixel instead of
+    # PyTorch's normalisation arithmetic).
+    unfolded = resnet18_var.ResNet18Var(masks=masks, precision=precision, fold_bn=False)
+    unfolded.load_state_dict(model.state_dict())
+    unfolded = unfolded.to(dev)
+    for c in unfolded.winograd_convs():
+        c.refresh()
+    assert rel_max(unfolded(image.to(dev)).cpu().numpy(), got) <= tol
