@@ -71,7 +71,7 @@ constexpr unsigned kOutOfRange = 0xfffffff0u;  // a byte offset no descriptor he
 
 // MF selects the MFMA shape of the asynchronous kernel: 32 = v_mfma_f32_32x32x2_f32 (16 accumulator
 // registers per tile), 16 = v_mfma_f32_16x16x4_f32 (4 registers per tile, 16-row granularity).
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int OCC_ = 2, int MF_ = 32>
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int OCC_ = 2, int MF_ = 32, int BPAD_ = -1>
 struct ConvCfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_, MF = MF_;
     static constexpr int OCC = OCC_;                     // waves per SIMD the register budget allows
@@ -81,6 +81,8 @@ struct ConvCfg {
     static constexpr int LG = 64 / MF;                   // lane groups: each feeds 4 reduction indices per operand read
     static constexpr int KG = 4 * LG;                    // reduction indices per operand group (4 MFMAs)
     static constexpr int REGS = MF * MF / 64;            // accumulator registers per tile
+    // Asynchronous kernel: floats of padding after every 4 rows (1 KiB) of the B tile in LDS.
+    static constexpr int BPAD = BPAD_ >= 0 ? BPAD_ : (MF == 16 ? 16 : 0);
     static constexpr int LDA = BK + 4;  // synchronous kernel: row stride (floats), 4*odd keeps b128 row reads conflict-free
     static constexpr int LDB = BN + 4;
     static constexpr int NA = BM * BK / (4 * NT);        // synchronous kernel: float4 per thread per A tile
@@ -415,7 +417,7 @@ __device__ __forceinline__ void wait_vmcnt()
 template <typename Cfg, int NSTAGE>
 constexpr int async_lds_bytes()
 {
-    constexpr int nbw = Cfg::BK * Cfg::BN / 4 / 64, bpad = Cfg::MF == 16 ? 16 : 0;
+    constexpr int nbw = Cfg::BK * Cfg::BN / 4 / 64, bpad = Cfg::BPAD;
     return NSTAGE * (Cfg::BM * Cfg::BK + Cfg::BK * Cfg::BN + nbw * bpad) * 4;
 }
 
@@ -438,7 +440,7 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     constexpr int NA = (NAW + NWAVES - 1) / NWAVES, NB = (NBW + NWAVES - 1) / NWAVES;
     // With 16x16 MFMAs the four lane groups of a B operand read hit rows 4 apart; 64 bytes of padding
     // after every copy (4 rows of 64 floats) put them on different banks.
-    constexpr int BPAD = MF == 16 ? 16 : 0;  // floats
+    constexpr int BPAD = Cfg::BPAD;  // floats
     static_assert(BPAD == 0 || BN == 64, "the padded B layout assumes one copy = 4 rows");
     constexpr int A_FLOATS = BM * BK, B_FLOATS = BK * BN + NBW * BPAD, STAGE_FLOATS = A_FLOATS + B_FLOATS;
     constexpr int LPS = NA + NB;  // copies per thread per step
