@@ -6,8 +6,11 @@
 // (winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans_grad_cuda.cu.cc:118-129).
 //
 // Conv grad keeps the reference's structure: dP = A dY A^T into the caller's 16*M*K temporary,
-// then two plain batched GEMMs (dTI = dP . W^T, dW = TI^T . dP), here rocBLAS strided-batched
-// SGEMM where the reference calls cublasSgemmBatched.  ImTrans grad is one gather kernel: every
+// then two batched GEMMs.  dTI = dP . W^T is a plain library GEMM (rocBLAS strided-batched SGEMM
+// where the reference calls cublasSgemmBatched).  dW = TI^T . dP reduces over the tens of thousands
+// of rows of M into a tiny output, a shape the library handles poorly (31 TFLOP/s at ResNet-18
+// conv3); it runs on the split-reduction MFMA kernel of winograd2x2_wgrad_kernel.h, with rocBLAS
+// kept for the shapes that kernel does not take.  ImTrans grad is one gather kernel: every
 // input pixel collects, from the up to 2x2 tiles that cover it, its entry of B dT B^T, recomputed
 // from the (at most 9) transform-domain gradients it depends on; the incoming gradient is not
 // modified (the reference transforms it in place first, :124).
@@ -17,6 +20,7 @@
 #include <rocblas/rocblas.h>
 
 #include "swc_common.h"
+#include "winograd2x2_wgrad_kernel.h"
 
 namespace swc {
 namespace {
@@ -148,6 +152,39 @@ rocblas_handle blas_handle()
     return handles[dev];
 }
 
+// dW through the split-reduction kernel.  The partial tiles of the S row splits are parked in the
+// dTI buffer, which the caller owns, which is at least S*16*C*K floats when S*K <= M, and which is
+// only written (in full) by the dTI GEMM that runs afterwards.  Returns SWC_ERR_UNSUPPORTED when the
+// shapes do not fit the kernel.
+int wgrad_own(const float *TI, const float *dP, float *dW, float *scratch, size_t M, int C, int K, hipStream_t s)
+{
+    if (M % WG_BK != 0 || C % 4 != 0 || K % 4 != 0 || !aligned16(TI) || !aligned16(dP) || !aligned16(dW) ||
+        !aligned16(scratch))
+        return SWC_ERR_UNSUPPORTED;
+    if (static_cast<size_t>(WG_BK) * C >= (1ull << 29) || static_cast<size_t>(WG_BK) * K >= (1ull << 29))
+        return SWC_ERR_UNSUPPORTED;  // 32-bit byte offsets within a tile
+    const size_t tiles_c = (static_cast<size_t>(C) + WG_BM - 1) / WG_BM, tiles_k = (static_cast<size_t>(K) + WG_BN - 1) / WG_BN;
+    const size_t base = 16 * tiles_c * tiles_k;
+    const size_t steps_total = M / WG_BK;
+    // Two workgroups per CU measured best (conv3: 61 us with 512 workgroups, 65-70 with 256 or 768+).
+    size_t S = base >= 512 ? 1 : (512 + base - 1) / base;
+    if (S > M / K) S = M / K;
+    if (S > steps_total) S = steps_total;
+    if (S < 1) S = 1;
+    const size_t per = (steps_total + S - 1) / S;
+    S = (steps_total + per - 1) / per;  // no empty split
+    if (S * base >= (1ull << 31)) return SWC_ERR_UNSUPPORTED;
+    const size_t nw = static_cast<size_t>(16) * C * K;
+    wgrad_splitk_kernel<<<dim3(static_cast<unsigned>(S * base)), dim3(256), WG_LDS_BYTES, s>>>(
+        TI, dP, S == 1 ? dW : scratch, M, C, K, static_cast<unsigned>(tiles_c), static_cast<unsigned>(tiles_k),
+        static_cast<unsigned>(per), static_cast<unsigned>(steps_total), nw);
+    int st = check_launch();
+    if (st != SWC_OK || S == 1) return st;
+    const unsigned n4 = static_cast<unsigned>(nw / 4);
+    wgrad_reduce_kernel<<<dim3((n4 + 255) / 256), dim3(256), 0, s>>>(scratch, dW, n4, static_cast<unsigned>(S), nw);
+    return check_launch();
+}
+
 }  // namespace
 }  // namespace swc
 
@@ -178,6 +215,11 @@ extern "C" int swc_winograd2x2_conv_grad(const float *TInput, const float *Weigh
     int st = check_launch();
     if (st != SWC_OK) return st;
 
+    // dW first: its partial sums borrow the dTI buffer before the dTI GEMM fills it.
+    st = wgrad_own(TInput, tmp_data_buffer, Weight_grad, TInput_grad, M, C, K, s);
+    const bool dw_done = st == SWC_OK;
+    if (!dw_done && st != SWC_ERR_UNSUPPORTED) return st;
+
     rocblas_handle h = blas_handle();
     if (h == nullptr || rocblas_set_stream(h, s) != rocblas_status_success) return SWC_ERR_HIP;
     const float one = 1.f, zero = 0.f;
@@ -189,6 +231,7 @@ extern "C" int swc_winograd2x2_conv_grad(const float *TInput, const float *Weigh
                                                       static_cast<rocblas_stride>(M) * K, &zero, TInput_grad, C,
                                                       static_cast<rocblas_stride>(M) * C, 16);
     if (rs != rocblas_status_success) return SWC_ERR_HIP;
+    if (dw_done) return SWC_OK;
     // Row-major dW[i] (C x K) = TI[i]^T . dP[i], as column-major (K x C) = (dP: K x M) . op_T(TI: C x M):
     // the call at winograd2x2_conv_grad_cuda.cu.cc:115-120.
     rs = rocblas_sgemm_strided_batched(h, rocblas_operation_none, rocblas_operation_transpose, K, C, Mi, &one,

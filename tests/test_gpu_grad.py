@@ -49,6 +49,10 @@ def test_imtrans_grad(oracle, dev, shape, masked):
 
 @pytest.mark.parametrize("shape", [
     (3, 3, 3, 32, 32), (2, 4, 4, 5, 7), (1, 1, 1, 1, 1), (2, 3, 5, 36, 100), (8, 14, 14, 128, 128),
+    # M % 32 == 0 takes the split-reduction weight-gradient kernel:
+    (2, 4, 4, 36, 100),   # one split, ragged channel and filter tiles
+    (16, 4, 4, 36, 20),   # 8 splits of a single step each
+    (6, 8, 8, 64, 72),    # 12 steps in 5 splits (3,3,3,3 -> per = 3, last split shorter)
 ])
 def test_conv_grad(oracle, dev, shape):
     from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv_grad
@@ -61,7 +65,7 @@ def test_conv_grad(oracle, dev, shape):
     dti, dw = winograd2x2_conv_grad(gpu(ti, dev), gpu(w, dev), gpu(dy, dev))
     assert rel_max(dti.cpu().numpy(), dti_want) <= TOL
     assert rel_max(dw.cpu().numpy(), dw_want) <= TOL
-    if B * nH * nW <= 64:
+    if B * nH * nW <= 384:
         tii = rng.integers(-3, 4, size=ti.shape).astype(np.float32)
         wi = rng.integers(-3, 4, size=w.shape).astype(np.float32)
         dyi = rng.integers(-3, 4, size=dy.shape).astype(np.float32)
