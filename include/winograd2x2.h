@@ -184,9 +184,12 @@ SWC_API int swc_winograd2x2_relu_conv(const float *Input, const float *Weight, f
  *   declared winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_grad_op.cc:32,
  *   defined  winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_grad_cuda.cu.cc:77-124.
  * tmp_data_buffer must hold 16*B*nH*nW*K floats (the caller's temporary, as at
- * winograd2x2_conv_grad_op.cc:69-71); tmp_ptr_buffer is ignored.  The two batched GEMMs run in
- * rocBLAS; the first call on a host thread creates that thread's rocBLAS handle, which is the one
- * piece of state (and device memory) this library ever owns.
+ * winograd2x2_conv_grad_op.cc:69-71); tmp_ptr_buffer is ignored.  TInput_grad is also used as
+ * scratch (partial sums of Weight_grad) before it receives its result, so it must not alias an input.
+ * The TInput_grad GEMM runs in rocBLAS (as does the Weight_grad GEMM for shapes the library's own
+ * kernel does not take: M % 32, C % 4, K % 4, alignment); the first call on a host thread creates
+ * that thread's rocBLAS handle, which is the one piece of state (and device memory) this library
+ * ever owns.
  */
 SWC_API int swc_winograd2x2_conv_grad(const float *TInput, const float *Weight, const float *Output_grad,
                                       float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,
