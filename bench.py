@@ -168,6 +168,8 @@ def main():
     ap.add_argument("--backward", action="store_true",
                     help="also time the two gradient ops (conv grad: dP transform + two rocBLAS batched GEMMs; "
                          "imTrans grad with the ReLU mask) and add a `backward` object to the line")
+    ap.add_argument("--graph", action="store_true",
+                    help="also replay the K steps from one captured HIP graph and report `ms_per_step_graph`")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run five 128 MiB device-to-device copies and exit: the known-size kernel that the "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled against")
@@ -250,6 +252,24 @@ def main():
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # The same K steps captured once into a HIP graph and replayed: what a caller whose loop is
+    # launch-bound would run (the launchers allocate nothing and never synchronise, so they capture).
+    ms_step_graph = None
+    if args.graph:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            cs = torch.cuda.current_stream().cuda_stream
+            for _ in range(args.steps):
+                if L.swc_winograd2x2_imtrans(xp, tip, C, B, H, W, 1, 1, 1, cs) != 0 or \
+                        conv_fn(tip, wp, yp, None, None, C, B, nH, nW, K, 1, 1, cs) != 0:
+                    raise RuntimeError("capture failed")
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        ms_step_graph = (time.perf_counter() - t0) * 1e3 / args.steps
+
     # Per-kernel average launch durations, HIP events on the launching (current) stream.
     ms_imtrans = time_loop(f_imtrans, args.steps, torch)
     ms_conv = time_loop(f_conv, args.steps, torch)
@@ -289,6 +309,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_step, 5),
+        "ms_per_step_graph": None if ms_step_graph is None else round(ms_step_graph, 5),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -351,3 +351,32 @@ def test_imtrans_affine_bit_exact(oracle, dev, shape, relu):
     # a non-zero shift must not leak into the padding: border tiles differ from transforming a padded-then-mapped image
     same = imtrans(gpu(oracle.affine(x, scale, shift), dev), relu=relu).cpu().numpy()
     assert np.array_equal(got, same)
+
+
+def test_forward_pair_replays_in_a_hip_graph(dev):
+    # The launchers allocate nothing and never synchronise, so imTrans + conv can be captured once and
+    # replayed; every replay (with eager work and synchronisations in between) must equal the eager result.
+    imtrans, conv = ops()
+    g = torch.Generator(device="cpu").manual_seed(77)
+    x = torch.randn(4, 14, 14, 64, generator=g).to(dev)
+    w = (torch.randn(16, 64, 96, generator=g) * 0.05).to(dev)
+    ti = torch.empty(16, 4, 7, 7, 64, device=dev)
+    y = torch.empty(4, 14, 14, 96, device=dev)
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        conv(imtrans(x, relu=True, out=ti), w, out=y)   # warm-up outside the capture
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        conv(imtrans(x, relu=True, out=ti), w, out=y)
+    for rep in range(4):
+        x.copy_(torch.randn(4, 14, 14, 64, generator=g))
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize(dev)
+        got = y.clone()
+        want = conv(imtrans(x, relu=True), w)           # eager work between replays
+        torch.cuda.synchronize(dev)
+        assert torch.equal(got, want), rep
