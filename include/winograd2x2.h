@@ -102,6 +102,22 @@ SWC_API int swc_winograd2x2_conv(const float *Input, const float *Weight, float 
                          swc_stream_t stream);
 
 /*
+ * swc_winograd2x2_conv with per-element work folded into its output stores:
+ *   Output = fmaf(conv, Scale[k], Shift[k]) + Residual
+ *   Scale, Shift [K] fp32 (both or neither); Residual [B,2nH,2nW,K] fp32; any of them may be NULL.
+ *   precision: 0 = fp32 MFMA, 1 = bf16 operands (as swc_winograd2x2_conv_bf16).
+ * No counterpart function in the reference: it is what follows its second convolution of every
+ * residual unit -- `BatchNorm('bn2a_2c', x)` at inference and the `tf.add([x, bra])` with the shortcut
+ * (ResNet-18-var/imagenet-resnet-transWino-prune.py:123,131 and the seven other units up to :213) --
+ * applied while the result is still in registers instead of in two more passes over it.
+ * Residual may alias Output (each element is read before it is written, by the same lane).
+ */
+SWC_API int swc_winograd2x2_conv_epilogue(const float *Input, const float *Weight, float *Output,
+                                  const float *Scale, const float *Shift, const float *Residual,
+                                  int C, int B, int nH, int nW, int K, int pad_h, int pad_w,
+                                  int precision, swc_stream_t stream);
+
+/*
  * Same contract as swc_winograd2x2_conv, with both GEMM operands rounded to bf16
  * (round-to-nearest-even) on their way into the matrix cores; accumulation and the
  * output transform stay fp32.  No counterpart in the reference (its GEMM is cuBLAS

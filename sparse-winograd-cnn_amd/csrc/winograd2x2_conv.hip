@@ -21,7 +21,8 @@ namespace {
 
 // Synchronous kernel: any shape and alignment (register-staged tiles, guarded or descriptor loads).
 template <typename Cfg, bool BF16>
-int launch_sync(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nH, int nW, hipStream_t stream)
+int launch_sync(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nH, int nW,
+                const ConvEpilogue &ep, hipStream_t stream)
 {
     const size_t tiles_m = (M + Cfg::BM - 1) / Cfg::BM;
     const size_t tiles_n = (static_cast<size_t>(K) + Cfg::BN - 1) / Cfg::BN;
@@ -32,10 +33,10 @@ int launch_sync(const float *TI, const float *Wt, float *Out, size_t M, int C, i
                       static_cast<size_t>(C) * K < (1ull << 29) && static_cast<size_t>(Cfg::BM) * C < (1ull << 29);
     if (fast)
         conv_mfma_kernel<Cfg, true, BF16><<<grid, block, 0, stream>>>(TI, Wt, Out, M, C, K, nH, nW,
-                                                                      static_cast<unsigned>(tiles_n));
+                                                                      static_cast<unsigned>(tiles_n), ep);
     else
         conv_mfma_kernel<Cfg, false, BF16><<<grid, block, 0, stream>>>(TI, Wt, Out, M, C, K, nH, nW,
-                                                                       static_cast<unsigned>(tiles_n));
+                                                                       static_cast<unsigned>(tiles_n), ep);
     return check_launch();
 }
 
@@ -51,7 +52,7 @@ bool async_eligible(const float *TI, const float *Wt, int C, int K)
 // rows_per_wg <= Cfg::BM rows of the [M,K] plane go to each workgroup.
 template <typename Cfg, int NSTAGE, bool BF16>
 int launch_async(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nH, int nW,
-                 size_t rows_per_wg, hipStream_t stream)
+                 size_t rows_per_wg, const ConvEpilogue &ep, hipStream_t stream)
 {
     constexpr int lds_bytes = async_lds_bytes<Cfg, NSTAGE>();
     static_assert(lds_bytes <= 64 * 1024, "larger tiles would need hipFuncAttributeMaxDynamicSharedMemorySize raised first");
@@ -60,7 +61,7 @@ int launch_async(const float *TI, const float *Wt, float *Out, size_t M, int C, 
     if (tiles_m * tiles_n >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
     const dim3 grid(static_cast<unsigned>(tiles_m * tiles_n)), block(Cfg::NT);
     conv_mfma_async_kernel<Cfg, NSTAGE, BF16><<<grid, block, lds_bytes, stream>>>(
-        TI, Wt, Out, M, C, K, nH, nW, static_cast<unsigned>(tiles_n), static_cast<unsigned>(rows_per_wg));
+        TI, Wt, Out, M, C, K, nH, nW, static_cast<unsigned>(tiles_n), static_cast<unsigned>(rows_per_wg), ep);
     return check_launch();
 }
 
@@ -90,9 +91,10 @@ size_t balanced_rows(size_t M, size_t tiles_n)
 
 template <bool BF16>
 int conv_entry(const float *Input, const float *Weight, float *Output, int C, int B, int nH, int nW, int K,
-               int pad_h, int pad_w, swc_stream_t stream)
+               int pad_h, int pad_w, const ConvEpilogue &ep, swc_stream_t stream)
 {
     if (Input == nullptr || Weight == nullptr || Output == nullptr) return SWC_ERR_NULL_POINTER;
+    if ((ep.scale == nullptr) != (ep.shift == nullptr)) return SWC_ERR_NULL_POINTER;
     if (C <= 0 || B <= 0 || nH <= 0 || nW <= 0 || K <= 0) return SWC_ERR_BAD_DIMS;
     if (pad_h != 1 || pad_w != 1) return SWC_ERR_BAD_PAD;
     const size_t M = static_cast<size_t>(B) * nH * nW;
@@ -120,25 +122,25 @@ int conv_entry(const float *Input, const float *Weight, float *Output, int C, in
         const double cost_short = ok_short ? passes((M + rows_short - 1) / rows_short * tiles_n) * 2.0 * (C >= 128 ? 0.98 : 1.15) : 1e30;
         if (ok_tall && cost_tall < cost32 && cost_tall <= cost_short) {
             note_conv_kernel("tall16");
-            return launch_async<Tall, 2, false>(Input, Weight, Output, M, C, K, nH, nW, rows_tall, s);
+            return launch_async<Tall, 2, false>(Input, Weight, Output, M, C, K, nH, nW, rows_tall, ep, s);
         }
         if (ok_short && cost_short < cost32) {
             note_conv_kernel("short16");
-            return launch_async<Short, 2, false>(Input, Weight, Output, M, C, K, nH, nW, rows_short, s);
+            return launch_async<Short, 2, false>(Input, Weight, Output, M, C, K, nH, nW, rows_short, ep, s);
         }
     }
     // Ring depth: the fp32 step is long (16 MFMAs of 64 cycles per wave) and one tile in flight
     // covers the memory latency; the bf16 step is 8x shorter and needs two.
     if (async_eligible<Tile32>(Input, Weight, C, K)) {
         note_conv_kernel("ring32");
-        return launch_async<Tile32, BF16 ? 3 : 2, BF16>(Input, Weight, Output, M, C, K, nH, nW, Tile32::BM, s);
+        return launch_async<Tile32, BF16 ? 3 : 2, BF16>(Input, Weight, Output, M, C, K, nH, nW, Tile32::BM, ep, s);
     }
     if (!BF16 && async_eligible<Tile16>(Input, Weight, C, K)) {
         note_conv_kernel("ring16");
-        return launch_async<Tile16, 3, false>(Input, Weight, Output, M, C, K, nH, nW, Tile16::BM, s);
+        return launch_async<Tile16, 3, false>(Input, Weight, Output, M, C, K, nH, nW, Tile16::BM, ep, s);
     }
     note_conv_kernel("sync");
-    return launch_sync<Tile32, BF16>(Input, Weight, Output, M, C, K, nH, nW, s);
+    return launch_sync<Tile32, BF16>(Input, Weight, Output, M, C, K, nH, nW, ep, s);
 }
 
 }  // namespace
@@ -147,12 +149,25 @@ int conv_entry(const float *Input, const float *Weight, float *Output, int C, in
 extern "C" int swc_winograd2x2_conv(const float *Input, const float *Weight, float *Output, float *, const long long *,
                                     int C, int B, int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream)
 {
-    return swc::conv_entry<false>(Input, Weight, Output, C, B, nH, nW, K, pad_h, pad_w, stream);
+    return swc::conv_entry<false>(Input, Weight, Output, C, B, nH, nW, K, pad_h, pad_w, swc::ConvEpilogue(), stream);
 }
 
 extern "C" int swc_winograd2x2_conv_bf16(const float *Input, const float *Weight, float *Output, float *,
                                          const long long *, int C, int B, int nH, int nW, int K, int pad_h, int pad_w,
                                          swc_stream_t stream)
 {
-    return swc::conv_entry<true>(Input, Weight, Output, C, B, nH, nW, K, pad_h, pad_w, stream);
+    return swc::conv_entry<true>(Input, Weight, Output, C, B, nH, nW, K, pad_h, pad_w, swc::ConvEpilogue(), stream);
+}
+
+extern "C" int swc_winograd2x2_conv_epilogue(const float *Input, const float *Weight, float *Output, const float *Scale,
+                                             const float *Shift, const float *Residual, int C, int B, int nH, int nW,
+                                             int K, int pad_h, int pad_w, int precision, swc_stream_t stream)
+{
+    swc::ConvEpilogue ep;
+    ep.scale = Scale;
+    ep.shift = Shift;
+    ep.residual = Residual;
+    if (precision == 0) return swc::conv_entry<false>(Input, Weight, Output, C, B, nH, nW, K, pad_h, pad_w, ep, stream);
+    if (precision == 1) return swc::conv_entry<true>(Input, Weight, Output, C, B, nH, nW, K, pad_h, pad_w, ep, stream);
+    return SWC_ERR_BAD_DIMS;
 }

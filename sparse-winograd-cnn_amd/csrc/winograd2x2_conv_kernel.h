@@ -95,6 +95,14 @@ struct ConvCfg {
 template <typename Cfg>
 using AccT = typename std::conditional<Cfg::MF == 32, floatx16, floatx4>::type;
 
+// Optional per-element work folded into the output stores: out = fmaf(y, scale[k], shift[k]) + residual.
+// scale and shift go together; either part may be absent (null).  All null: plain stores.
+struct ConvEpilogue {
+    const float *scale = nullptr;     // [K]
+    const float *shift = nullptr;     // [K]
+    const float *residual = nullptr;  // [B,2nH,2nW,K], the output's layout
+};
+
 // Scatter of the four output tiles: tile row m = (b*nH + th)*nW + tw -> pixels (2th+dy, 2tw+dx)
 // of image b (winograd2x2_conv_cuda.cu.cc:48-51).  Accumulator register r of lane (lg, li) holds
 // column li and row 8*(r/4) + 4*lg + r%4 of a 32x32 tile, row 4*lg + r of a 16x16 tile.  Only the
@@ -103,9 +111,10 @@ using AccT = typename std::conditional<Cfg::MF == 32, floatx16, floatx4>::type;
 template <typename Cfg>
 __device__ __forceinline__ void store_output(const AccT<Cfg> (&Y)[4][Cfg::TM][Cfg::TN], float *__restrict__ Out,
                                              unsigned rows_valid, int K, int nW, size_t m0, int n0, int wm0, int wn0,
-                                             int li, int lg)
+                                             int li, int lg, const ConvEpilogue ep = ConvEpilogue())
 {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, MF = Cfg::MF;
+    const bool affine = ep.scale != nullptr, residual = ep.residual != nullptr;  // uniform over the grid
     const size_t oW = 2 * static_cast<size_t>(nW);
     const size_t row_stride = oW * K;
     const unsigned m032 = static_cast<unsigned>(m0);
@@ -118,15 +127,31 @@ __device__ __forceinline__ void store_output(const AccT<Cfg> (&Y)[4][Cfg::TM][Cf
             const unsigned gm = m032 + row;
             const unsigned bt = gm / static_cast<unsigned>(nW);  // b*nH + th
             const unsigned tw = gm - bt * static_cast<unsigned>(nW);
-            float *o = Out + (static_cast<size_t>(bt) * 2 * oW + 2 * tw) * K;
+            const size_t pix = (static_cast<size_t>(bt) * 2 * oW + 2 * tw) * K;
+            float *o = Out + pix;
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
                 const int col = n0 + wn0 + tn * MF + li;
                 if (col >= K) continue;
-                o[col] = Y[0][tm][tn][r];
-                o[K + col] = Y[1][tm][tn][r];
-                o[row_stride + col] = Y[2][tm][tn][r];
-                o[row_stride + K + col] = Y[3][tm][tn][r];
+                float y0 = Y[0][tm][tn][r], y1 = Y[1][tm][tn][r], y2 = Y[2][tm][tn][r], y3 = Y[3][tm][tn][r];
+                if (affine) {
+                    const float sc = ep.scale[col], sh = ep.shift[col];
+                    y0 = __builtin_fmaf(y0, sc, sh);
+                    y1 = __builtin_fmaf(y1, sc, sh);
+                    y2 = __builtin_fmaf(y2, sc, sh);
+                    y3 = __builtin_fmaf(y3, sc, sh);
+                }
+                if (residual) {
+                    const float *q = ep.residual + pix;
+                    y0 += q[col];
+                    y1 += q[K + col];
+                    y2 += q[row_stride + col];
+                    y3 += q[row_stride + K + col];
+                }
+                o[col] = y0;
+                o[K + col] = y1;
+                o[row_stride + col] = y2;
+                o[row_stride + K + col] = y3;
             }
         }
     }
@@ -141,7 +166,7 @@ __device__ __forceinline__ void store_output(const AccT<Cfg> (&Y)[4][Cfg::TM][Cf
 template <typename Cfg, bool FAST, bool BF16>
 __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_mfma_kernel(
     const float *__restrict__ TI, const float *__restrict__ Wt, float *__restrict__ Out, size_t M, int C, int K, int nH,
-    int nW, unsigned tiles_n)
+    int nW, unsigned tiles_n, ConvEpilogue ep)
 {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, LDA = Cfg::LDA, LDB = Cfg::LDB, NA = Cfg::NA, NB = Cfg::NB;
@@ -349,7 +374,7 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
                 for (int tn = 0; tn < TN; ++tn) asm volatile("" : "+v"(Y[j][tm][tn]));
     }
 
-    store_output<Cfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg);
+    store_output<Cfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -428,7 +453,7 @@ constexpr int async_lds_bytes()
 template <typename Cfg, int NSTAGE, bool BF16 = false, int ABL = 0>
 __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_mfma_async_kernel(
     const float *__restrict__ TI, const float *__restrict__ Wt, float *__restrict__ Out, size_t M, int C, int K, int nH,
-    int nW, unsigned tiles_n, unsigned rows_per_wg)
+    int nW, unsigned tiles_n, unsigned rows_per_wg, ConvEpilogue ep)
 {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT, MF = Cfg::MF, LG = Cfg::LG, KG = Cfg::KG;
     constexpr int TM = Cfg::TM, TN = Cfg::TN;
@@ -724,7 +749,7 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     // The surplus copies must have landed before this workgroup's LDS can be handed on.
     wait_vmcnt<0>();
 
-    if (!(ABL & 16) || nH < 0) store_output<Cfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg);
+    if (!(ABL & 16) || nH < 0) store_output<Cfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
 }
 
 }  // namespace

@@ -13,7 +13,8 @@ after, not before).
 Everything except the two Winograd ops is stock PyTorch.  Activations are kept NHWC in memory
 (channels_last), so handing them to the ops and back costs no copies.  The BatchNorm in front of
 each WinogradImTrans (inference statistics) is folded into the transform kernel as a per-channel
-scale and shift; ``fold_bn=False`` runs it as its own pass instead.
+scale and shift, and the BatchNorm plus residual add behind each unit's second convolution into
+that convolution's stores; ``fold_bn=False`` runs them as separate PyTorch passes instead.
 """
 import os
 import sys
@@ -83,23 +84,26 @@ class WinogradUnit(torch.nn.Module):
             self.conv1 = torch.nn.Conv2d(c_in, c_out, 1, bias=False)
             self.bn1 = torch.nn.BatchNorm2d(c_out)
 
-    def branch(self, x):
+    def branch(self, x, shortcut=None):
+        """The two Winograd layers.  With ``fold_bn`` the three BatchNorms and the residual add run inside
+        the Winograd kernels (bn2a, bn2b in the transforms' loads; bn2c and ``+ shortcut`` in the second
+        convolution's stores) and the result is already ``shortcut + branch``."""
         if self.fold_bn:
             h = self.conv2a(WinogradImTrans(_to_nhwc(x), torch.relu, affine=_bn_affine(self.bn2a)))
-            h = self.conv2b(WinogradImTrans(h, torch.relu, affine=_bn_affine(self.bn2b)))
-            return self.bn2c(_to_nchw(h))
+            h = self.conv2b(WinogradImTrans(h, torch.relu, affine=_bn_affine(self.bn2b)),
+                            affine=_bn_affine(self.bn2c), residual=_to_nhwc(shortcut))
+            return _to_nchw(h)
         h = _to_nchw(self.conv2a(WinogradImTrans(_to_nhwc(self.bn2a(x)), torch.relu)))
         h = _to_nchw(self.conv2b(WinogradImTrans(_to_nhwc(self.bn2b(h)), torch.relu)))
-        return self.bn2c(h)
+        return shortcut + self.bn2c(h)
 
     def forward(self, x):
-        bra = self.branch(x)
         if self.shortcut:
             s = torch.relu(self.bn_pre(x)) if self.bn_pre is not None else torch.relu(x)
-            x = self.bn1(self.conv1(s))
+            sc = self.bn1(self.conv1(s))
         else:
-            x = torch.relu(x)
-        x = x + bra
+            sc = torch.relu(x)
+        x = self.branch(x, sc)
         if self.pool:
             x = F.max_pool2d(F.pad(x, _same_pad(x, 3, 2), value=float("-inf")), 3, 2)
         return x

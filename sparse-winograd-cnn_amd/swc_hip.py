@@ -22,6 +22,7 @@ SWC_ERR_UNSUPPORTED = -6
 C_SYMBOLS = (
     "swc_strerror", "swc_last_hip_error", "swc_version", "swc_winograd2x2_conv_last_kernel",
     "swc_winograd2x2_imtrans", "swc_winograd2x2_imtrans_affine", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
+    "swc_winograd2x2_conv_epilogue",
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
     "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad", "swc_winograd2x2_relu_conv",
@@ -77,6 +78,8 @@ def lib():
         for f in (L.swc_winograd2x2_conv, L.swc_winograd2x2_conv_bf16):
             f.restype = i32
             f.argtypes = [fp, fp, fp, fp, vp] + [i32] * 7 + [vp]
+        L.swc_winograd2x2_conv_epilogue.restype = i32
+        L.swc_winograd2x2_conv_epilogue.argtypes = [fp] * 6 + [i32] * 8 + [vp]
         L.swc_winograd2x2_imtrans_op_shape.restype = i32
         L.swc_winograd2x2_imtrans_op_shape.argtypes = [i32, i64p, i64p]
         L.swc_winograd2x2_imtrans_op_compute.restype = i32

@@ -24,7 +24,7 @@ def winograd2x2_conv_shape(i_shape, w_shape):
     return tuple(out)
 
 
-def _forward(I, W, precision, out):
+def _forward(I, W, precision, out, scale=None, shift=None, residual=None):
     if precision not in PRECISIONS:
         raise ValueError("precision must be one of %s" % sorted(PRECISIONS))
     I = swc_hip.require_cuda_f32(I, "I", 5)
@@ -37,11 +37,30 @@ def _forward(I, W, precision, out):
     else:
         if tuple(out.shape) != shape or out.dtype != torch.float32 or out.device != I.device or not out.is_contiguous():
             raise ValueError("out must be a contiguous float32 tensor of shape %s on %s" % (shape, I.device))
+    if (scale is None) != (shift is None):
+        raise ValueError("scale and shift go together")
+    epilogue = scale is not None or residual is not None
+    if scale is not None:
+        scale = swc_hip.require_cuda_f32(scale, "scale", 1)
+        shift = swc_hip.require_cuda_f32(shift, "shift", 1)
+        if scale.shape[0] != shape[3] or shift.shape[0] != shape[3]:
+            raise ValueError("scale and shift must have one entry per output channel (%d)" % shape[3])
+    if residual is not None:
+        residual = swc_hip.require_cuda_f32(residual, "residual", 4)
+        if tuple(residual.shape) != shape:
+            raise ValueError("residual must have the output's shape %s" % (shape,))
     with torch.cuda.device(I.device):
         stream = torch.cuda.current_stream().cuda_stream
-        st = swc_hip.lib().swc_winograd2x2_conv_op_compute(
-            I.data_ptr(), 5, swc_hip.dims(I.shape), W.data_ptr(), 3, swc_hip.dims(W.shape),
-            out.data_ptr(), 4, swc_hip.dims(out.shape), PRECISIONS[precision], stream)
+        if epilogue:
+            _, B, nH, nW, C = I.shape
+            st = swc_hip.lib().swc_winograd2x2_conv_epilogue(
+                I.data_ptr(), W.data_ptr(), out.data_ptr(), None if scale is None else scale.data_ptr(),
+                None if shift is None else shift.data_ptr(), None if residual is None else residual.data_ptr(),
+                C, B, nH, nW, shape[3], 1, 1, PRECISIONS[precision], stream)
+        else:
+            st = swc_hip.lib().swc_winograd2x2_conv_op_compute(
+                I.data_ptr(), 5, swc_hip.dims(I.shape), W.data_ptr(), 3, swc_hip.dims(W.shape),
+                out.data_ptr(), 4, swc_hip.dims(out.shape), PRECISIONS[precision], stream)
     swc_hip.check(st, "winograd2x2_conv")
     return out
 
@@ -83,16 +102,22 @@ class _ConvFunction(torch.autograd.Function):
         return dI, dW, None
 
 
-def winograd2x2_conv(I, W, precision="fp32", out=None):
+def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, residual=None):
     """I: [16,B,nH,nW,C], W: [16,C,K], float32 on the GPU -> [B,2nH,2nW,K] (uncropped).
+
+    ``scale``/``shift`` ([K]) and ``residual`` ([B,2nH,2nW,K]), forward only: the result becomes
+    ``conv*scale + shift + residual`` inside the kernel's stores (an inference BatchNorm and the
+    residual add that follow the second convolution of a ResNet unit).
 
     ``precision="bf16"`` rounds both GEMM operands to bf16 (fp32 accumulate).  Differentiable
     through ``winograd2x2_conv_grad`` when an input requires grad.
     """
     needs_grad = torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (I, W))
+    if (scale is not None or residual is not None) and needs_grad:
+        raise NotImplementedError("the scale/shift/residual epilogue is forward only")
     if out is None and needs_grad:
         return _ConvFunction.apply(I, W, precision)
-    return _forward(I, W, precision, out)
+    return _forward(I, W, precision, out, scale, shift, residual)
 
 
 def winograd2x2_relu_conv(X, W, relu=True, out=None):

@@ -58,9 +58,13 @@ class WinogradConv(torch.nn.Module):
             self._masked = (self.W.data * self.mask).contiguous()
         return self._masked
 
-    def forward(self, x):
+    def forward(self, x, affine=None, residual=None):
+        """``affine=(scale, shift)`` and ``residual`` (forward only) are applied to the result inside
+        the kernel: ``conv*scale + shift + residual``."""
         if torch.is_grad_enabled() and self.W.requires_grad:
             w = self.W if self.mask is None else self.W * self.mask
         else:
             w = self.masked_weight()
-        return winograd2x2_conv.winograd2x2_conv.winograd2x2_conv(x, w, precision=self.precision)
+        scale, shift = affine if affine is not None else (None, None)
+        return winograd2x2_conv.winograd2x2_conv.winograd2x2_conv(x, w, precision=self.precision, scale=scale,
+                                                                  shift=shift, residual=residual)

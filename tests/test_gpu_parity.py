@@ -380,3 +380,40 @@ def test_forward_pair_replays_in_a_hip_graph(dev):
         want = conv(imtrans(x, relu=True), w)           # eager work between replays
         torch.cuda.synchronize(dev)
         assert torch.equal(got, want), rep
+
+
+@pytest.mark.parametrize("shape", [(3, 3, 3, 32, 32), (2, 4, 4, 5, 7), (8, 9, 9, 128, 72), (16, 14, 14, 128, 128),
+                                   (1, 5, 7, 48, 20)])
+@pytest.mark.parametrize("parts", ["affine", "residual", "both"])
+def test_conv_epilogue(oracle, dev, shape, parts):
+    # Output = fmaf(conv, scale, shift) + residual inside the stores, on every kernel the launcher picks.
+    _, conv = ops()
+    B, nH, nW, C, K = shape
+    ti, w = conv_inputs(shape, 21)
+    rng = np.random.default_rng(22)
+    scale = (0.5 + rng.random(K)).astype(np.float32) * rng.choice([-1, 1], K).astype(np.float32)
+    shift = rng.standard_normal(K).astype(np.float32)
+    res = rng.standard_normal((B, 2 * nH, 2 * nW, K)).astype(np.float32)
+    plain = conv(gpu(ti, dev), gpu(w, dev))
+    kw, want = {}, plain.cpu().numpy()
+    if parts in ("affine", "both"):
+        kw.update(scale=gpu(scale, dev), shift=gpu(shift, dev))
+        want = oracle.affine(want, scale, shift)
+    if parts in ("residual", "both"):
+        kw.update(residual=gpu(res, dev))
+        want = want + res
+    got = conv(gpu(ti, dev), gpu(w, dev), **kw).cpu().numpy()
+    # same kernel, same accumulators: the epilogue arithmetic itself is exact against the oracle's
+    assert np.array_equal(got, want)
+    # and the whole thing against the float64-accumulated oracle
+    full = oracle.conv(ti, w, acc64=True).astype(np.float64)
+    if parts in ("affine", "both"):
+        full = full * scale + shift
+    if parts in ("residual", "both"):
+        full = full + res
+    assert rel_max(got, full) <= TOL
+    # in place: residual aliasing the output
+    if parts == "residual":
+        buf = gpu(res, dev)
+        conv(gpu(ti, dev), gpu(w, dev), out=buf, residual=buf)
+        assert np.array_equal(buf.cpu().numpy(), want)

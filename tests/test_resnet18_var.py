@@ -55,8 +55,13 @@ def test_forward_matches_oracle_path(oracle, precision, tol):
             x = oracle.affine(x, affine[0].detach().numpy(), affine[1].detach().numpy())
         return torch.from_numpy(oracle.imtrans(x, relu=True))
 
-    def cpu_conv_forward(self, x):
-        return torch.from_numpy(oracle.conv(x.numpy(), self.masked_weight().numpy(), acc64=True))
+    def cpu_conv_forward(self, x, affine=None, residual=None):
+        y = oracle.conv(x.numpy(), self.masked_weight().numpy(), acc64=True)
+        if affine is not None:
+            y = oracle.affine(y, affine[0].detach().numpy(), affine[1].detach().numpy())
+        if residual is not None:
+            y = y + residual.numpy()
+        return torch.from_numpy(y)
 
     orig_imtrans, orig_forward = resnet18_var.WinogradImTrans, winograd_conv.WinogradConv.forward
     try:
