@@ -110,16 +110,20 @@ int conv_entry(const float *Input, const float *Weight, float *Output, int C, in
     using Short = ConvCfg<32, 64, 64, 1, 4, 3, 16>;
     if (!BF16) {
         // Cost = passes x MFMA work of a wave per pass (in 16x16 tiles), weighted by what each kernel
-        // measured per unit of that work on MI355X relative to Tile32 (Tall 8 % more; Short about
-        // equal when its 64-channel steps are at least two per position, 15 % more otherwise).
+        // measured per unit of that work on MI355X relative to Tile32, over the ResNet-18 shapes at
+        // batch 64 and 128: Tall 8 % more; Short 10 % more, 15 % more when its 64-channel steps are
+        // fewer than two per position, but 3 % less while all of its workgroups are resident at once
+        // (up to three per CU).
         const size_t tiles_n = (static_cast<size_t>(K) + 63) / 64;
         const bool ok32 = async_eligible<Tile32>(Input, Weight, C, K);
         const bool ok_tall = async_eligible<Tall>(Input, Weight, C, K);
         const bool ok_short = async_eligible<Short>(Input, Weight, C, K);
         const size_t rows_tall = balanced_rows<Tall>(M, tiles_n), rows_short = balanced_rows<Short>(M, tiles_n);
+        const size_t wgs_short = (M + rows_short - 1) / rows_short * tiles_n;
+        const double w_short = C < 128 ? 1.15 : wgs_short <= 3 * kCUs ? 0.97 : 1.10;
         const double cost32 = ok32 ? passes((M + 63) / 64 * tiles_n) * 4.0 : 1e30;
         const double cost_tall = ok_tall ? passes((M + rows_tall - 1) / rows_tall * tiles_n) * 7.0 * 1.08 : 1e30;
-        const double cost_short = ok_short ? passes((M + rows_short - 1) / rows_short * tiles_n) * 2.0 * (C >= 128 ? 0.98 : 1.15) : 1e30;
+        const double cost_short = ok_short ? passes(wgs_short) * 2.0 * w_short : 1e30;
         if (ok_tall && cost_tall < cost32 && cost_tall <= cost_short) {
             note_conv_kernel("tall16");
             return launch_async<Tall, 2, false>(Input, Weight, Output, M, C, K, nH, nW, rows_tall, ep, s);
