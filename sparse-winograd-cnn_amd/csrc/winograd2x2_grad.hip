@@ -72,73 +72,97 @@ __global__ __launch_bounds__(256) void output_transform_grad_kernel(const float 
 
 // ---- dX = col2im(B dT B^T) (+ ReLU mask) ----------------------------------------------------------
 // Along one axis, pixel y lies in tile y/2 and in one neighbour; with patch offset r = y + 1 - 2*tile,
-// (B dT B^T)[r][.] = sum_u BT[u][r] dT[u][.], BT = [[1,0,-1,0],[0,1,1,0],[0,-1,1,0],[0,1,0,-1]]:
-//   r=0: +u0        r=1: +u1 -u2 +u3        r=2: -u0 +u1 +u2        r=3: -u3
-struct AxisTerms {
-    int tile[4], u[4];
-    float sign[4];  // 0 marks a term outside the tile grid
-};
-__device__ __forceinline__ AxisTerms axis_terms(int y, int n_tiles)
-{
-    AxisTerms o;
-    const int t = y >> 1;
-    if (y & 1) {  // r = 2 in tile t, r = 0 in tile t+1
-        o.tile[0] = t; o.u[0] = 0; o.sign[0] = -1.f;
-        o.tile[1] = t; o.u[1] = 1; o.sign[1] = 1.f;
-        o.tile[2] = t; o.u[2] = 2; o.sign[2] = 1.f;
-        const bool ok = t + 1 < n_tiles;
-        o.tile[3] = ok ? t + 1 : t; o.u[3] = 0; o.sign[3] = ok ? 1.f : 0.f;
-    } else {      // r = 1 in tile t, r = 3 in tile t-1
-        o.tile[0] = t; o.u[0] = 1; o.sign[0] = 1.f;
-        o.tile[1] = t; o.u[1] = 2; o.sign[1] = -1.f;
-        o.tile[2] = t; o.u[2] = 3; o.sign[2] = 1.f;
-        const bool ok = t >= 1;
-        o.tile[3] = ok ? t - 1 : t; o.u[3] = 3; o.sign[3] = ok ? -1.f : 0.f;
-    }
-    return o;
-}
-
+// (B dT B^T)[r][.] = sum_u BT[u][r] dT[u][.], BT = [[1,0,-1,0],[0,1,1,0],[0,-1,1,0],[0,1,0,-1]].
+// A gather, one lane per (tile, VEC channels) producing the tile's four interior pixels
+// (2th+a, 2tw+b), a, b in {0,1}.  Pixel (a,b) sits at patch offset (1+a, 1+b) of its own tile, at row
+// 3 / 0 of the tile above / below (a = 0 / 1), at column 3 / 0 of the tile to the left / right
+// (b = 0 / 1), and at a corner of the diagonal neighbour.  With
+//   row(r)[v] = sum_u BT[u][r] dT[u][v]   (r=0: +u0   r=1: +u1 -u2 +u3   r=2: -u0 +u1 +u2   r=3: -u3)
+// and the same combination over v for the column, the own tile needs all 16 planes once, each edge
+// neighbour one row or column of 4 planes and each corner one plane: 36 loads for 4 pixels where the
+// per-pixel form issues 64.
 template <int VEC, bool MASK>
-__global__ __launch_bounds__(256) void imtrans_grad_kernel(const float *__restrict__ dT, const float *__restrict__ mask_src,
-                                                           float *__restrict__ dX, int H, int W, int C, int nH, int nW,
-                                                           unsigned items, size_t plane)
+__global__ __launch_bounds__(256) void imtrans_grad_tile_kernel(const float *__restrict__ dT,
+                                                                const float *__restrict__ mask_src,
+                                                                float *__restrict__ dX, int H, int W, int C, int nH,
+                                                                int nW, unsigned items, size_t plane)
 {
     using V = typename GVec<VEC>::type;
     const unsigned idx = xcd_swizzle(blockIdx.x, gridDim.x) * 256 + threadIdx.x;
     if (idx >= items) return;
     const unsigned CV = C / VEC;
     const unsigned cv = idx % CV;
-    unsigned p = idx / CV;
-    const int x = p % W;
-    p /= W;
-    const int y = p % H;
-    const unsigned b = p / H;
-    const AxisTerms ry = axis_terms(y, nH), rx = axis_terms(x, nW);
-    float acc[VEC];
+    unsigned m = idx / CV;
+    const int tw = m % nW;
+    m /= nW;
+    const int th = m % nH;
+    const unsigned b = m / nH;
+    // masked gradient of plane 4u+v at tile (th+dy, tw+dx), zero outside the tile grid
+    auto g = [&](int u, int v, int dy, int dx) __attribute__((always_inline)) -> V {
+        const size_t off = static_cast<size_t>(4 * u + v) * plane +
+                           ((static_cast<size_t>(b) * nH + (th + dy)) * nW + (tw + dx)) * C + static_cast<size_t>(cv) * VEC;
+        V x = *reinterpret_cast<const V *>(dT + off);
+        if (MASK) {
+            const V t = *reinterpret_cast<const V *>(mask_src + off);
+            float *xp = reinterpret_cast<float *>(&x);
+            const float *tp = reinterpret_cast<const float *>(&t);
 #pragma unroll
-    for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float sg = ry.sign[i] * rx.sign[j];
-            const size_t off = static_cast<size_t>(4 * ry.u[i] + rx.u[j]) * plane +
-                               ((static_cast<size_t>(b) * nH + ry.tile[i]) * nW + rx.tile[j]) * C + static_cast<size_t>(cv) * VEC;
-            const V g = *reinterpret_cast<const V *>(dT + off);
-            const float *gp = reinterpret_cast<const float *>(&g);
-            if (MASK) {
-                const V t = *reinterpret_cast<const V *>(mask_src + off);
-                const float *tp = reinterpret_cast<const float *>(&t);
-#pragma unroll
-                for (int q = 0; q < VEC; ++q) acc[q] += (sg != 0.f && tp[q] > 0.f) ? sg * gp[q] : 0.f;
-            } else {
-#pragma unroll
-                for (int q = 0; q < VEC; ++q) acc[q] += sg != 0.f ? sg * gp[q] : 0.f;
-            }
+            for (int q = 0; q < VEC; ++q) xp[q] = tp[q] > 0.f ? xp[q] : 0.f;
         }
-    float *o = dX + static_cast<size_t>(idx) * VEC;
+        return x;
+    };
+    // combination over one axis: offset 1 -> +e1 -e2 +e3, offset 2 -> -e0 +e1 +e2
+    auto mid = [](int a, V e0, V e1, V e2, V e3) __attribute__((always_inline)) -> V {
+        return a == 0 ? add(sub(e1, e2), e3) : add(sub(e1, e0), e2);
+    };
+    const bool up = th > 0, down = th + 1 < nH, left = tw > 0, right = tw + 1 < nW;
+    V out[2][2];
+    {   // own tile: rows 1+a, then columns 1+b
+        V row[2][4];
 #pragma unroll
-    for (int q = 0; q < VEC; ++q) o[q] = acc[q];
+        for (int v = 0; v < 4; ++v) {
+            const V e0 = g(0, v, 0, 0), e1 = g(1, v, 0, 0), e2 = g(2, v, 0, 0), e3 = g(3, v, 0, 0);
+            row[0][v] = mid(0, e0, e1, e2, e3);
+            row[1][v] = mid(1, e0, e1, e2, e3);
+        }
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int bb = 0; bb < 2; ++bb) out[a][bb] = mid(bb, row[a][0], row[a][1], row[a][2], row[a][3]);
+    }
+    if (up) {      // row 3 of the tile above: -dT[3][v]
+        const V e0 = g(3, 0, -1, 0), e1 = g(3, 1, -1, 0), e2 = g(3, 2, -1, 0), e3 = g(3, 3, -1, 0);
+        out[0][0] = sub(out[0][0], mid(0, e0, e1, e2, e3));
+        out[0][1] = sub(out[0][1], mid(1, e0, e1, e2, e3));
+    }
+    if (down) {    // row 0 of the tile below: +dT[0][v]
+        const V e0 = g(0, 0, 1, 0), e1 = g(0, 1, 1, 0), e2 = g(0, 2, 1, 0), e3 = g(0, 3, 1, 0);
+        out[1][0] = add(out[1][0], mid(0, e0, e1, e2, e3));
+        out[1][1] = add(out[1][1], mid(1, e0, e1, e2, e3));
+    }
+    if (left) {    // column 3 of the tile to the left: -dT[u][3]
+        const V e0 = g(0, 3, 0, -1), e1 = g(1, 3, 0, -1), e2 = g(2, 3, 0, -1), e3 = g(3, 3, 0, -1);
+        out[0][0] = sub(out[0][0], mid(0, e0, e1, e2, e3));
+        out[1][0] = sub(out[1][0], mid(1, e0, e1, e2, e3));
+    }
+    if (right) {   // column 0 of the tile to the right: +dT[u][0]
+        const V e0 = g(0, 0, 0, 1), e1 = g(1, 0, 0, 1), e2 = g(2, 0, 0, 1), e3 = g(3, 0, 0, 1);
+        out[0][1] = add(out[0][1], mid(0, e0, e1, e2, e3));
+        out[1][1] = add(out[1][1], mid(1, e0, e1, e2, e3));
+    }
+    // corners: (-1)(-1) dT[3][3], (-1)(+1) dT[3][0], (+1)(-1) dT[0][3], (+1)(+1) dT[0][0]
+    if (up && left) out[0][0] = add(out[0][0], g(3, 3, -1, -1));
+    if (up && right) out[0][1] = sub(out[0][1], g(3, 0, -1, 1));
+    if (down && left) out[1][0] = sub(out[1][0], g(0, 3, 1, -1));
+    if (down && right) out[1][1] = add(out[1][1], g(0, 0, 1, 1));
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int bb = 0; bb < 2; ++bb) {
+            const int y = 2 * th + a, x = 2 * tw + bb;
+            if (y < H && x < W)
+                *reinterpret_cast<V *>(dX + ((static_cast<size_t>(b) * H + y) * W + x) * C + static_cast<size_t>(cv) * VEC) = out[a][bb];
+        }
 }
 
 // ---- rocBLAS handle: one per host thread and device, created on first use -------------------------
@@ -255,11 +279,12 @@ extern "C" int swc_winograd2x2_imtrans_grad(const float *TransIm_grad, const flo
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool vec = (C % 4 == 0) && aligned16(TransIm_grad) && aligned16(Input_grad) &&
                      (relu_mask_source == nullptr || aligned16(relu_mask_source));
-    const unsigned items = static_cast<unsigned>(pixels * (vec ? C / 4 : C));
+    // one lane per (tile, channel vector): each writes the four pixels its tile is centred on
+    const unsigned items = static_cast<unsigned>(static_cast<size_t>(B) * nH * nW * (vec ? C / 4 : C));
     const dim3 grid((items + 255) / 256), block(256);
-#define SWC_LAUNCH(VEC, MASK)                                                                                        \
-    imtrans_grad_kernel<VEC, MASK><<<grid, block, 0, s>>>(TransIm_grad, relu_mask_source, Input_grad, H, W, C, nH, nW, \
-                                                          items, plane)
+#define SWC_LAUNCH(VEC, MASK)                                                                                   \
+    imtrans_grad_tile_kernel<VEC, MASK><<<grid, block, 0, s>>>(TransIm_grad, relu_mask_source, Input_grad, H, W, C, \
+                                                               nH, nW, items, plane)
     if (vec) {
         if (relu_mask_source) SWC_LAUNCH(4, true); else SWC_LAUNCH(4, false);
     } else {
