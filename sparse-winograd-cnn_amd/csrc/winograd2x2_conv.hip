@@ -55,7 +55,20 @@ int launch_async(const float *TI, const float *Wt, float *Out, size_t M, int C, 
                  size_t rows_per_wg, const ConvEpilogue &ep, hipStream_t stream)
 {
     constexpr int lds_bytes = async_lds_bytes<Cfg, NSTAGE>();
-    static_assert(lds_bytes <= 64 * 1024, "larger tiles would need hipFuncAttributeMaxDynamicSharedMemorySize raised first");
+    static_assert(lds_bytes <= 160 * 1024, "a CU has 160 KiB of LDS");
+    if (lds_bytes > 64 * 1024) {
+        // Above the default 64 KiB limit, which is raised once per kernel and device.
+        constexpr int kMaxDevices = 64;
+        static thread_local bool raised[kMaxDevices] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return SWC_ERR_HIP;
+        if (!raised[dev]) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(conv_mfma_async_kernel<Cfg, NSTAGE, BF16>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+            if (e != hipSuccess) return note_hip_error(e);
+            raised[dev] = true;
+        }
+    }
     const size_t tiles_m = (M + rows_per_wg - 1) / rows_per_wg;
     const size_t tiles_n = (static_cast<size_t>(K) + Cfg::BN - 1) / Cfg::BN;
     if (tiles_m * tiles_n >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
