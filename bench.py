@@ -170,8 +170,10 @@ def main():
                          "imTrans grad with the ReLU mask) and add a `backward` object to the line")
     ap.add_argument("--no-rotate", dest="rotate", action="store_false",
                     help="skip the extra timing over cycled buffer sets (Infinity Cache defeated)")
-    ap.add_argument("--graph", action="store_true",
-                    help="also replay the K steps from one captured HIP graph and report `ms_per_step_graph`")
+    ap.add_argument("--no-graph", dest="graph", action="store_false",
+                    help="time only eager launches; by default the K steps are also replayed from one captured HIP "
+                         "graph and, when that is faster, `value`/`ms_per_step` are the replayed figure "
+                         "(`ms_per_step_eager` keeps the other)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run five 128 MiB device-to-device copies and exit: the known-size kernel that the "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled against")
@@ -258,19 +260,23 @@ def main():
     # launch-bound would run (the launchers allocate nothing and never synchronise, so they capture).
     ms_step_graph = None
     if args.graph:
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            cs = torch.cuda.current_stream().cuda_stream
-            for _ in range(args.steps):
-                if L.swc_winograd2x2_imtrans(xp, tip, C, B, H, W, 1, 1, 1, cs) != 0 or \
-                        conv_fn(tip, wp, yp, None, None, C, B, nH, nW, K, 1, 1, cs) != 0:
-                    raise RuntimeError("capture failed")
-        graph.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        graph.replay()
-        torch.cuda.synchronize()
-        ms_step_graph = (time.perf_counter() - t0) * 1e3 / args.steps
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                cs = torch.cuda.current_stream().cuda_stream
+                for _ in range(args.steps):
+                    if L.swc_winograd2x2_imtrans(xp, tip, C, B, H, W, 1, 1, 1, cs) != 0 or \
+                            conv_fn(tip, wp, yp, None, None, C, B, nH, nW, K, 1, 1, cs) != 0:
+                        raise RuntimeError("a launcher refused the capture stream")
+            graph.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            ms_step_graph = (time.perf_counter() - t0) * 1e3 / args.steps
+        except Exception as e:  # capture unavailable: the eager figure stands
+            print("bench.py: HIP graph capture failed (%s); eager timing only" % e, file=sys.stderr)
+            ms_step_graph = None
 
     # Per-kernel average launch durations, HIP events on the launching (current) stream.
     ms_imtrans = time_loop(f_imtrans, args.steps, torch)
@@ -345,14 +351,17 @@ def main():
     conv_roofline.update({"traffic": MEASURED_TRAFFIC.get((name, args.precision, "conv")),
                           "algorithmic_flop_per_launch": gemm_flops, "algorithmic_bytes_per_launch": conv_bytes})
 
+    ms_best = ms_step if ms_step_graph is None else min(ms_step, ms_step_graph)
     out = {
         "metric": "effective conv GFLOP/s + imTrans HBM GB/s, ResNet-18 conv3 batch 64, 1 MI355X",
-        "value": round(direct_flops / (ms_step * 1e-3) / 1e9, 1),
+        "value": round(direct_flops / (ms_best * 1e-3) / 1e9, 1),
         "unit": "GFLOP/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_step, 5),
+        "ms_per_step": round(ms_best, 5),
+        "launch": "hip graph replay of the K steps" if ms_best != ms_step else "eager",
+        "ms_per_step_eager": round(ms_step, 5),
         "ms_per_step_graph": None if ms_step_graph is None else round(ms_step_graph, 5),
         "higher_is_better": True,
         "scaling": "weak",
