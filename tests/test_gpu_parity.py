@@ -417,3 +417,51 @@ def test_conv_epilogue(oracle, dev, shape, parts):
         buf = gpu(res, dev)
         conv(gpu(ti, dev), gpu(w, dev), out=buf, residual=buf)
         assert np.array_equal(buf.cpu().numpy(), want)
+
+
+def test_channels_beyond_the_reference_block_limit(oracle, dev):
+    # The reference launches one thread per channel (block = C, winograd2x2_imTrans_cuda.cu.cc:154) or per
+    # filter (block = K, winograd2x2_conv_cuda.cu.cc:87), so it stops at 1024; these kernels do not.
+    imtrans, conv = ops()
+    rng = np.random.default_rng(41)
+    x = rng.standard_normal((1, 4, 6, 2052)).astype(np.float32)
+    assert np.array_equal(imtrans(gpu(x, dev), relu=True).cpu().numpy(), oracle.imtrans(x, relu=True))
+    ti, w = conv_inputs((1, 2, 3, 64, 1100), 42)
+    got = conv(gpu(ti, dev), gpu(w, dev)).cpu().numpy()
+    assert rel_max(got, oracle.conv(ti, w, acc64=True)) <= TOL
+
+
+def test_host_threads_on_their_own_streams(oracle, dev):
+    # The launchers keep no shared mutable state: four host threads, each on its own stream with its own
+    # tensors, must all get the result a single thread gets.
+    import threading
+    imtrans, conv = ops()
+    shapes = [(2, 10, 10, 64, 64), (3, 6, 6, 32, 32), (2, 7, 9, 48, 20), (4, 14, 14, 128, 72)]
+    inputs, wants, gots, errors = [], [], [None] * 4, []
+    for i, (B, H, W, C, K) in enumerate(shapes):
+        rng = np.random.default_rng(50 + i)
+        x = rng.standard_normal((B, H, W, C)).astype(np.float32)
+        w = (rng.standard_normal((16, C, K)) * 0.05).astype(np.float32)
+        inputs.append((gpu(x, dev), gpu(w, dev)))
+        wants.append(oracle.conv(oracle.imtrans(x, relu=True), w, acc64=True))
+    torch.cuda.synchronize(dev)
+
+    def work(i):
+        try:
+            stream = torch.cuda.Stream(device=dev)
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    y = conv(imtrans(inputs[i][0], relu=True), inputs[i][1])
+                stream.synchronize()
+                gots[i] = y.cpu().numpy()
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for got, want in zip(gots, wants):
+        assert rel_max(got, want) <= TOL
