@@ -147,7 +147,8 @@ def bench_resnet(args, torch, dev):
         "value": round(flops / (ms * 1e-3) / 1e9, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": steps,
         "warmup": max(args.warmup // 4, 2), "ms_per_step": round(ms, 3), "images_per_s": round(N / (ms * 1e-3), 1),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if args.precision == "fp32" else "bf16 operands, f32 accumulate", "data": "synthetic",
+        "dtype": {"fp32": "f32", "bf16": "bf16 operands, f32 accumulate",
+                  "bf16_stored": "bf16 operands (stored as bf16), f32 accumulate"}[args.precision], "data": "synthetic",
         "config": {"workload": "cfg5: ResNet-18-var forward, N=%d, 224x224x3, whole model time incl. stock "
                                "PyTorch conv1/1x1/BN/pool/FC" % N, "gemm_precision": args.precision},
         "logits_finite": bool(torch.isfinite(logits).all()),
@@ -162,7 +163,9 @@ def main():
     ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg5"],
                     help="cfg1-cfg4b: one layer; cfg5: the whole ResNet-18-var forward (16 Winograd layers), N=128")
     ap.add_argument("--batch", type=int, default=128, help="batch size of the cfg5 forward")
-    ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16"])
+    ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16", "bf16_stored"],
+                    help="fp32 (the reference's arithmetic); bf16: GEMM operands rounded to bf16 inside the conv "
+                         "kernel; bf16_stored: the transformed activations are also written and read as bf16")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg and the parity gate")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU work for cpu_baseline")
     ap.add_argument("--backward", action="store_true",
@@ -216,7 +219,8 @@ def main():
     x_np, w_np = make_inputs(name)
     x = torch.from_numpy(x_np).to(dev)
     w = torch.from_numpy(w_np).to(dev)
-    ti = torch.empty(16, B, nH, nW, C, device=dev)
+    stored = args.precision == "bf16_stored"
+    ti = torch.empty(16, B, nH, nW, C, device=dev, dtype=torch.bfloat16 if stored else torch.float32)
     y = torch.empty(B, 2 * nH, 2 * nW, K, device=dev)
 
     # The timed loop calls the launcher-level C entry points directly with prebuilt arguments
@@ -224,18 +228,37 @@ def main():
     # than the transform kernel runs for).  The wrappers are exercised once, for the record.
     L = swc_hip.lib()
     stream = torch.cuda.current_stream().cuda_stream
-    conv_fn = L.swc_winograd2x2_conv if args.precision == "fp32" else L.swc_winograd2x2_conv_bf16
     xp, wp, tip, yp = x.data_ptr(), w.data_ptr(), ti.data_ptr(), y.data_ptr()
-    winograd2x2_imTrans(x, relu=True, out=ti)
-    winograd2x2_conv(ti, w, precision=args.precision, out=y)
+    if stored:
+        from winograd2x2_conv.winograd2x2_conv import winograd2x2_weights_bf16
+        w16 = winograd2x2_weights_bf16(w)   # prepared once, like W*mask
+        w16p = w16.data_ptr()
+        winograd2x2_imTrans(x, relu=True, out=ti, out_dtype=torch.bfloat16)
+        winograd2x2_conv(ti, w16, out=y)
+
+        def call_imtrans(a, b, st):
+            return L.swc_winograd2x2_imtrans_bf16out(a, None, None, b, C, B, H, W, 1, 1, 1, st)
+
+        def call_conv(b, c, st):
+            return L.swc_winograd2x2_conv_bf16in(b, w16p, c, None, None, None, C, B, nH, nW, K, 1, 1, st)
+    else:
+        conv_entry = L.swc_winograd2x2_conv if args.precision == "fp32" else L.swc_winograd2x2_conv_bf16
+        winograd2x2_imTrans(x, relu=True, out=ti)
+        winograd2x2_conv(ti, w, precision=args.precision, out=y)
+
+        def call_imtrans(a, b, st):
+            return L.swc_winograd2x2_imtrans(a, b, C, B, H, W, 1, 1, 1, st)
+
+        def call_conv(b, c, st):
+            return conv_entry(b, wp, c, None, None, C, B, nH, nW, K, 1, 1, st)
 
     def f_imtrans():
-        if L.swc_winograd2x2_imtrans(xp, tip, C, B, H, W, 1, 1, 1, stream) != 0:
-            raise RuntimeError("swc_winograd2x2_imtrans failed")
+        if call_imtrans(xp, tip, stream) != 0:
+            raise RuntimeError("the imTrans launcher failed")
 
     def f_conv():
-        if conv_fn(tip, wp, yp, None, None, C, B, nH, nW, K, 1, 1, stream) != 0:
-            raise RuntimeError("swc_winograd2x2_conv failed")
+        if call_conv(tip, yp, stream) != 0:
+            raise RuntimeError("the conv launcher failed")
 
     def step():
         f_imtrans()
@@ -265,8 +288,7 @@ def main():
             with torch.cuda.graph(graph):
                 cs = torch.cuda.current_stream().cuda_stream
                 for _ in range(args.steps):
-                    if L.swc_winograd2x2_imtrans(xp, tip, C, B, H, W, 1, 1, 1, cs) != 0 or \
-                            conv_fn(tip, wp, yp, None, None, C, B, nH, nW, K, 1, 1, cs) != 0:
+                    if call_imtrans(xp, tip, cs) != 0 or call_conv(tip, yp, cs) != 0:
                         raise RuntimeError("a launcher refused the capture stream")
             graph.replay()
             torch.cuda.synchronize()
@@ -287,12 +309,12 @@ def main():
     # The same kernels over buffer sets that are cycled, so that consecutive launches cannot be served
     # from the 256 MB Infinity Cache: together the sets are larger than it.
     rotated = None
-    set_bytes = (x.numel() + ti.numel() + y.numel()) * 4
+    set_bytes = (x.numel() + y.numel()) * 4 + ti.numel() * ti.element_size()
     n_sets = max(2, -(-3 * 256 * 2 ** 20 // set_bytes)) if args.rotate else 0
     if n_sets and n_sets * set_bytes < 64 * 2 ** 30:
         sets = [(x.clone(), torch.empty_like(ti), torch.empty_like(y)) for _ in range(n_sets)]
         for xs, ts, ys in sets:
-            winograd2x2_imTrans(xs, relu=True, out=ts)
+            call_imtrans(xs.data_ptr(), ts.data_ptr(), stream)
         ptrs = [(a.data_ptr(), b.data_ptr(), c.data_ptr()) for a, b, c in sets]
         state = {"i": 0}
 
@@ -302,18 +324,17 @@ def main():
 
         def r_imtrans():
             a, b, _ = nxt()
-            if L.swc_winograd2x2_imtrans(a, b, C, B, H, W, 1, 1, 1, stream) != 0:
-                raise RuntimeError("swc_winograd2x2_imtrans failed")
+            if call_imtrans(a, b, stream) != 0:
+                raise RuntimeError("the imTrans launcher failed")
 
         def r_conv():
             _, b, c = nxt()
-            if conv_fn(b, wp, c, None, None, C, B, nH, nW, K, 1, 1, stream) != 0:
-                raise RuntimeError("swc_winograd2x2_conv failed")
+            if call_conv(b, c, stream) != 0:
+                raise RuntimeError("the conv launcher failed")
 
         def r_step():
             a, b, c = nxt()
-            if L.swc_winograd2x2_imtrans(a, b, C, B, H, W, 1, 1, 1, stream) != 0 or \
-                    conv_fn(b, wp, c, None, None, C, B, nH, nW, K, 1, 1, stream) != 0:
+            if call_imtrans(a, b, stream) != 0 or call_conv(b, c, stream) != 0:
                 raise RuntimeError("step failed")
 
         for f in (r_imtrans, r_conv, r_step):
@@ -330,8 +351,9 @@ def main():
 
     direct_flops = 18.0 * B * H * W * C * K
     gemm_flops = 32.0 * M * C * K
-    imtrans_bytes = 4.0 * B * H * W * C + 64.0 * M * C
-    conv_bytes = 64.0 * M * C + 64.0 * C * K + 16.0 * M * K
+    ti_el = 2.0 if stored else 4.0   # bytes per element of TI (and of the weights the conv reads)
+    imtrans_bytes = 4.0 * B * H * W * C + 16.0 * ti_el * M * C
+    conv_bytes = 16.0 * ti_el * M * C + 16.0 * ti_el * C * K + 16.0 * M * K
     tf_conv = gemm_flops / (ms_conv * 1e-3) / 1e12
     gbs_imtrans = imtrans_bytes / (ms_imtrans * 1e-3) / 1e9
     gbs_conv = conv_bytes / (ms_conv * 1e-3) / 1e9
@@ -341,8 +363,9 @@ def main():
                          "achieved": round(tf_conv, 2), "peak": FP32_MFMA_PEAK_TF, "unit": "TFLOP/s",
                          "frac": round(tf_conv / FP32_MFMA_PEAK_TF, 4)}
     else:
-        # with bf16 operands the ridge is ~310 flop/B: every ResNet-18 shape is bound by reading the fp32 TI
-        conv_roofline = {"kernel": "winograd2x2_conv (16 GEMMs + fused A^T m A), bf16 MFMA", "bound": "hbm",
+        # with bf16 operands the ridge is ~310 flop/B: every ResNet-18 shape is bound by reading TI
+        conv_roofline = {"kernel": "winograd2x2_conv (16 GEMMs + fused A^T m A), bf16 MFMA, %s TI"
+                                   % ("bf16-stored" if stored else "fp32-stored"), "bound": "hbm",
                          "achieved": round(gbs_conv, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs_conv / HBM_PEAK_GBS, 4),
                          "mfma_TFLOPs": round(tf_conv, 2), "mfma_peak_TFLOPs": BF16_MFMA_PEAK_TF}
@@ -366,7 +389,8 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32" if args.precision == "fp32" else "bf16 operands, f32 accumulate",
+        "dtype": {"fp32": "f32", "bf16": "bf16 operands, f32 accumulate",
+                  "bf16_stored": "bf16 operands (stored as bf16), f32 accumulate"}[args.precision],
         "data": "synthetic",
         "config": {
             "workload": "%s: winograd2x2_imTrans(+ReLU) + winograd2x2_conv, N=%d %dx%dx%d -> %d, fp32 NHWC, "
@@ -441,9 +465,14 @@ def main():
         out["cpu_baseline"] = cpu
         # Parity gate on the very buffers that were timed.
         import oracle
-        ti_gpu = ti.cpu().numpy()
+        ti_gpu = ti.float().cpu().numpy()
         y_gpu = y.cpu().numpy()
-        y_ref = oracle.conv(ti_ref, w_np, acc64=True)
+        if stored:   # the transform is rounded once to bf16 as it is stored; the weights once when prepared
+            ti_ref = oracle.round_bf16(ti_ref)
+            y_ref = oracle.conv(ti_ref, oracle.round_bf16(w_np), acc64=True)
+            y32_ref = oracle.conv(ti_ref, oracle.round_bf16(w_np))
+        else:
+            y_ref = oracle.conv(ti_ref, w_np, acc64=True)
         den = float(np.max(np.abs(y_ref)))
         out["parity"] = {
             "imtrans_bit_exact": bool(np.array_equal(ti_gpu, ti_ref)),

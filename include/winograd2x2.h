@@ -187,6 +187,32 @@ SWC_API int swc_winograd2x2_relu_conv(const float *Input, const float *Weight, f
                                       int relu, swc_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * bf16-stored variant of the forward pair (no counterpart in the reference, whose tensors are all
+ * fp32): the transformed activations are written, kept and read as bf16, which halves the traffic of
+ * the HBM-bound half of the path.  Arithmetic: the transform and its ReLU in fp32 exactly as in
+ * swc_winograd2x2_imtrans, one rounding to bf16 (nearest even) on the store; the GEMMs multiply the
+ * bf16 operands exactly and accumulate in fp32; output transform and output in fp32 -- the same
+ * values swc_winograd2x2_conv_bf16 computes from the fp32 TransIm.
+ * ------------------------------------------------------------------------- */
+
+/* swc_winograd2x2_imtrans (Scale == Shift == NULL) or swc_winograd2x2_imtrans_affine, with
+ * TransIm16 [16,B,nH,nW,C] stored as bf16 bit patterns. */
+SWC_API int swc_winograd2x2_imtrans_bf16out(const float *Input, const float *Scale, const float *Shift,
+                                    uint16_t *TransIm16, int C, int B, int H, int W, int pad_h, int pad_w,
+                                    int relu, swc_stream_t stream);
+
+/* Weight [16,C,K] fp32 -> Weight16t [16,K,C] bf16 (nearest even), the layout the kernel below reads.
+ * Done once per weight update, like the W*mask of ResNet-18-var/winograd_conv.py:25. */
+SWC_API int swc_winograd2x2_weights_bf16(const float *Weight, uint16_t *Weight16t, int C, int K, swc_stream_t stream);
+
+/* swc_winograd2x2_conv_epilogue over the bf16 operands: Output [B,2nH,2nW,K] fp32 =
+ * fmaf(conv, Scale[k], Shift[k]) + Residual (Scale/Shift/Residual may be NULL).  Needs C % 64 == 0 and
+ * 16-byte aligned operands; returns SWC_ERR_UNSUPPORTED otherwise (use the fp32-stored path). */
+SWC_API int swc_winograd2x2_conv_bf16in(const uint16_t *Input16, const uint16_t *Weight16t, float *Output,
+                                const float *Scale, const float *Shift, const float *Residual, int C, int B,
+                                int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Backward ops.
  * ------------------------------------------------------------------------- */
 

@@ -92,6 +92,18 @@ def imtrans_affine(x, scale, shift, relu=False):
     return imtrans(affine(x, scale, shift), relu=relu)
 
 
+def round_bf16(a):
+    """fp32 -> nearest bf16 (ties to even), returned widened back to fp32.  Finite inputs only."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32).reshape(np.shape(a))
+
+
+def bf16_bits(a):
+    """The 16-bit patterns of round_bf16(a)."""
+    return (round_bf16(a).view(np.uint32) >> 16).astype(np.uint16)
+
+
 def gemm16(ti, w, acc64=False):
     """ti [16,M,C] (any leading tile dims), w [16,C,K] -> P [16,M,K] fp32."""
     ti, tp = _f32(ti)

@@ -1,0 +1,190 @@
+// Winograd convolution over bf16-stored operands for gfx950: the 16 GEMMs
+// P_i [M,K] = TI_i [M,C] . W_i [C,K] with TI held in memory as bf16 [16,M,C] and the weights as
+// bf16, transposed, [16,K,C]; fp32 accumulation, fp32 output transform and fp32 output, as in
+// conv_mfma_async_kernel.  Same arithmetic as swc_winograd2x2_conv_bf16 (operands rounded to bf16,
+// products exact in fp32), with the rounding done once by whoever wrote the operands instead of in
+// this kernel's registers, and half the bytes to move: the path is HBM-bound.
+//
+// Both operands have the reduction index (channels) as their fast axis, so both LDS tiles are
+// [64 rows][64 channels = 128 bytes = 8 chunks of 16 bytes] and an MFMA operand
+// (v_mfma_f32_32x32x16_bf16: lane (li, lg) holds 8 consecutive channels 8*lg.. of row li) is one
+// ds_read_b128 with no conversion.  Chunk c of row r is stored at slot c ^ (r % 8): the 32 lanes of
+// an operand read then spread over all banks.
+#pragma once
+
+#include "winograd2x2_conv_kernel.h"
+
+namespace swc {
+namespace {
+
+constexpr int HB_BM = 64, HB_BN = 64;  // tile of the [M,K] plane; 4 waves, 2x2, 32x32 each
+using HbStoreCfg = ConvCfg<HB_BM, HB_BN, 32, 2, 2>;
+
+// BK channels per step (a tile row is BK*2 bytes = CH chunks of 16), NSTAGE ring slots, OCC waves per SIMD.
+template <int BK_, int NSTAGE_, int OCC_>
+struct HbCfg {
+    static constexpr int BK = BK_, NSTAGE = NSTAGE_, OCC = OCC_;
+    static constexpr int CH = BK / 8;                    // 16-byte chunks per tile row
+    static constexpr int ROWS_PER_COPY = 64 / CH;        // rows one wave-wide copy (1 KiB) covers
+    static constexpr int TILE_BYTES = 64 * BK * 2;       // per operand
+    static constexpr int TILE_COPIES = TILE_BYTES / 1024;
+    static constexpr int PER_WAVE = TILE_COPIES / 4;     // copies of each tile per wave and step
+    static constexpr int COPIES = 2 * PER_WAVE;          // per thread and step
+    static constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
+    static constexpr int NMFMA = BK / 16;                // MFMAs per step and wave
+    static_assert(BK == 32 || BK == 64 || BK == 128, "a tile row is 4, 8 or 16 chunks");
+    static_assert(TILE_COPIES % 4 == 0, "every wave issues the same number of copies");
+    static_assert((NSTAGE - 2) * COPIES < 64, "vmcnt range");
+};
+
+// Requires C % BK == 0 and 16-byte aligned TI16 / Wt16.  M < 2^31.
+// ABL: timing ablations for development (bit 0: no barrier, 1: no copy wait, 2: no copies, 3: no LDS
+// reads, 4: no MFMA); results are wrong with any bit set.  Always 0 in the library.
+template <typename Cfg, int ABL = 0>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_bf16_stored_kernel(
+    const unsigned short *__restrict__ TI16, const unsigned short *__restrict__ Wt16, float *__restrict__ Out, size_t M,
+    int C, int K, int nH, int nW, unsigned tiles_n, ConvEpilogue ep)
+{
+    constexpr int BK = Cfg::BK, NSTAGE = Cfg::NSTAGE, CH = Cfg::CH, RPC = Cfg::ROWS_PER_COPY, PW = Cfg::PER_WAVE;
+    constexpr int ROW_BYTES = BK * 2;
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem_b[];
+
+    const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
+    const size_t m0 = static_cast<size_t>(lid / tiles_n) * HB_BM;
+    const int n0 = static_cast<int>(lid % tiles_n) * HB_BN;
+    const unsigned rows_valid = static_cast<unsigned>(M - m0 < HB_BM ? M - m0 : HB_BM);
+    const unsigned cols_valid = static_cast<unsigned>(K - n0 < HB_BN ? K - n0 : HB_BN);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lg = lane >> 5;
+    const int wm0 = static_cast<int>(wave >> 1) * 32, wn0 = static_cast<int>(wave & 1) * 32;
+    const int nkc = C / BK;
+
+    // ---- copies: wave-copy wl of a tile covers its rows RPC*wl .. RPC*wl+RPC-1 (1 KiB) ------------------
+    // Rows beyond the valid ones re-read the last valid row; they only reach outputs that are never stored.
+    unsigned a_voff[PW], b_voff[PW], t_lds[PW];
+#pragma unroll
+    for (int q = 0; q < PW; ++q) {
+        const unsigned wl = wave * PW + q;
+        const unsigned row = RPC * wl + lane / CH, slot = lane % CH, chunk = slot ^ (row % CH);
+        const unsigned ra = row < rows_valid ? row : rows_valid - 1, rb = row < cols_valid ? row : cols_valid - 1;
+        a_voff[q] = (ra * static_cast<unsigned>(C) + chunk * 8) * 2u;
+        b_voff[q] = (rb * static_cast<unsigned>(C) + chunk * 8) * 2u;
+        t_lds[q] = wl * 1024u;
+    }
+    const unsigned smem_base = lds_address(smem_b);
+    const size_t a_pos_stride = M * static_cast<size_t>(C), b_pos_stride = static_cast<size_t>(K) * C;
+    const unsigned short *a_pos = TI16 + m0 * C, *b_pos = Wt16 + static_cast<size_t>(n0) * C;
+    const unsigned short *a_next = a_pos, *b_next = b_pos;
+    int kc_next = 0, pos_next = 0;
+    unsigned slot_next = 0;
+    // Every thread issues exactly Cfg::COPIES copies per call; past the last step the walk wraps to
+    // position 0 again (copied, never read).
+    auto issue = [&]() __attribute__((always_inline)) {
+        const unsigned dst = smem_base + slot_next * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int q = 0; q < PW; ++q) async_copy16(reinterpret_cast<const float *>(a_next), a_voff[q], dst + t_lds[q]);
+#pragma unroll
+        for (int q = 0; q < PW; ++q)
+            async_copy16(reinterpret_cast<const float *>(b_next), b_voff[q], dst + Cfg::TILE_BYTES + t_lds[q]);
+        if (++kc_next == nkc) {
+            kc_next = 0;
+            if (++pos_next == 16) {
+                pos_next = 0;
+                a_pos = TI16 + m0 * C;
+                b_pos = Wt16 + static_cast<size_t>(n0) * C;
+            } else {
+                a_pos += a_pos_stride;
+                b_pos += b_pos_stride;
+            }
+            a_next = a_pos;
+            b_next = b_pos;
+        } else {
+            a_next += BK;
+            b_next += BK;
+        }
+        slot_next = slot_next + 1 == NSTAGE ? 0 : slot_next + 1;
+    };
+
+    floatx16 Y[4][1][1];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) Y[j][0][0][r] = 0.f;
+
+#pragma unroll
+    for (int i = 0; i < NSTAGE - 1; ++i) issue();
+
+    // byte offsets of this lane's operand chunks within a stage: MFMA h of a step takes chunk 2h + lg
+    unsigned a_off[Cfg::NMFMA], b_off[Cfg::NMFMA];
+#pragma unroll
+    for (int h = 0; h < Cfg::NMFMA; ++h) {
+        const unsigned ra = wm0 + li, rb = wn0 + li;
+        a_off[h] = ra * ROW_BYTES + (((2 * h + lg) ^ (ra % CH)) * 16u);
+        b_off[h] = Cfg::TILE_BYTES + rb * ROW_BYTES + (((2 * h + lg) ^ (rb % CH)) * 16u);
+    }
+    unsigned st_cur = 0;
+
+    static_for<16>([&](auto pos_tag) {
+        constexpr int pos = decltype(pos_tag)::value;
+        floatx16 P = {};
+        for (int kc = 0; kc < nkc; ++kc) {
+            // Step's tiles have landed once at most the copies of the NSTAGE-2 steps after it are
+            // outstanding; after the barrier everyone is also done with the slot the next copies overwrite.
+            if (!(ABL & 2)) wait_vmcnt<(NSTAGE - 2) * Cfg::COPIES>();
+            if (!(ABL & 1)) __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            if (!(ABL & 4)) issue();
+            bf16x8 a[Cfg::NMFMA], b[Cfg::NMFMA];
+#pragma unroll
+            for (int h = 0; h < Cfg::NMFMA; ++h) {
+                if (ABL & 8) {
+                    a[h] = bf16x8{};
+                    b[h] = bf16x8{};
+                    asm volatile("" : "+v"(a[h]), "+v"(b[h]));
+                } else {
+                    a[h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_cur + a_off[h]);
+                    b[h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_cur + b_off[h]);
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < Cfg::NMFMA; ++h) {
+                if (ABL & 16) {
+                    P[h] += static_cast<float>(a[h][0]) + static_cast<float>(b[h][0]);
+                } else {
+                    P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[h], b[h], P, 0, 0, 0);
+                }
+            }
+            st_cur = st_cur + Cfg::STAGE_BYTES == Cfg::LDS_BYTES ? 0 : st_cur + Cfg::STAGE_BYTES;
+        }
+        // fold P_pos into the running output tiles, ascending pos (winograd2x2_conv_cuda.cu.cc:39-46)
+        constexpr unsigned long long plus = kPlus, minus = kMinus;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if ((plus >> (4 * pos + j)) & 1ull)
+                Y[j][0][0] += P;
+            else if ((minus >> (4 * pos + j)) & 1ull)
+                Y[j][0][0] -= P;
+        }
+    });
+    wait_vmcnt<0>();  // the surplus copies must land before the workgroup's LDS is handed on
+
+    store_output<HbStoreCfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
+}
+
+// W [16,C,K] fp32 -> Wt16 [16,K,C] bf16 (round to nearest even).  One lane per output element.
+__global__ __launch_bounds__(256) void weights_to_bf16_transposed_kernel(const float *__restrict__ W,
+                                                                         unsigned short *__restrict__ Wt16, int C, int K,
+                                                                         unsigned n)
+{
+    const unsigned idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const unsigned c = idx % C, k = (idx / C) % K, pos = idx / (static_cast<unsigned>(C) * K);
+    const float v = round_bf16(W[(static_cast<size_t>(pos) * C + c) * K + k]);
+    Wt16[idx] = static_cast<unsigned short>(__float_as_uint(v) >> 16);
+}
+
+}  // namespace
+}  // namespace swc

@@ -77,6 +77,19 @@ __device__ __forceinline__ void stream_store(float *p, const float4 &v)
     __builtin_nontemporal_store(t, reinterpret_cast<floatx4_t *>(p));
 }
 
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned pack_bf16(float lo, float hi)
+{
+    const bf16x2_t p = __builtin_convertvector(floatx2_t{lo, hi}, bf16x2_t);  // v_cvt_pk_bf16_f32, RNE
+    return __builtin_bit_cast(unsigned, p);
+}
+__device__ __forceinline__ void store_bf16(unsigned short *p, float v) { *p = static_cast<unsigned short>(pack_bf16(v, 0.f)); }
+__device__ __forceinline__ void store_bf16(unsigned short *p, const float4 &v)
+{
+    *reinterpret_cast<uint2 *>(p) = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
+}
+
 template <int VEC, bool RELU>
 __device__ __forceinline__ void transform_vec(const typename Vec<VEC>::type (&d)[16], typename Vec<VEC>::type (&t)[16])
 {
@@ -103,7 +116,7 @@ __device__ __forceinline__ void transform_vec(const typename Vec<VEC>::type (&d)
 // AFFINE: every pixel inside the image is first mapped to fma(x, scale[c], shift[c]) (an inference-mode
 // batch normalisation folded into the load); the zero padding stays zero, as it does when the
 // normalisation runs as its own pass before the transform.
-template <int VEC, bool RELU, bool AFFINE, bool STREAM, typename Idx>
+template <int VEC, bool RELU, bool AFFINE, bool STREAM, bool BF16OUT, typename Idx>
 __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__restrict__ X, float *__restrict__ TI,
                                                              const float *__restrict__ scale,
                                                              const float *__restrict__ shift, int H, int W, int C,
@@ -153,6 +166,13 @@ __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__rest
     }
     V t[16];
     transform_vec<VEC, RELU>(d, t);
+    if (BF16OUT) {
+        // the planes are stored as bf16 (round to nearest even): TI is then [16,B,nH,nW,C] of 2-byte elements
+        unsigned short *dst16 = reinterpret_cast<unsigned short *>(TI) + static_cast<size_t>(idx) * VEC;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) store_bf16(dst16 + i * plane, t[i]);
+        return;
+    }
     float *dst = TI + static_cast<size_t>(idx) * VEC;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -178,24 +198,27 @@ bool use_stream_stores(size_t out_bytes)
 
 template <int VEC, bool RELU, bool AFFINE, typename Idx>
 int launch_direct(const float *X, const float *scale, const float *shift, float *TI, int B, int H, int W, int C, int nH,
-                  int nW, hipStream_t stream)
+                  int nW, bool bf16_out, hipStream_t stream)
 {
     const size_t M = static_cast<size_t>(B) * nH * nW;
     const size_t items = M * (C / VEC);
     const size_t blocks = (items + 255) / 256;
     const dim3 grid(static_cast<unsigned>(blocks)), block(256);
-    if (use_stream_stores(16 * M * C * sizeof(float)))
-        imtrans_direct_kernel<VEC, RELU, AFFINE, true, Idx><<<grid, block, 0, stream>>>(
+    if (bf16_out)
+        imtrans_direct_kernel<VEC, RELU, AFFINE, false, true, Idx><<<grid, block, 0, stream>>>(
+            X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
+    else if (use_stream_stores(16 * M * C * sizeof(float)))
+        imtrans_direct_kernel<VEC, RELU, AFFINE, true, false, Idx><<<grid, block, 0, stream>>>(
             X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
     else
-        imtrans_direct_kernel<VEC, RELU, AFFINE, false, Idx><<<grid, block, 0, stream>>>(
+        imtrans_direct_kernel<VEC, RELU, AFFINE, false, false, Idx><<<grid, block, 0, stream>>>(
             X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
     return check_launch();
 }
 
 template <bool AFFINE>
 int imtrans_entry(const float *Input, const float *Scale, const float *Shift, float *TransIm, int C, int B, int H, int W,
-                  int pad_h, int pad_w, int relu, swc_stream_t stream)
+                  int pad_h, int pad_w, int relu, bool bf16_out, swc_stream_t stream)
 {
     if (Input == nullptr || TransIm == nullptr) return SWC_ERR_NULL_POINTER;
     if (AFFINE && (Scale == nullptr || Shift == nullptr)) return SWC_ERR_NULL_POINTER;
@@ -206,12 +229,14 @@ int imtrans_entry(const float *Input, const float *Scale, const float *Shift, fl
     // One lane per item, 256 per workgroup, grid.x below 2^31.
     if (M * C / 256 >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool vec = (C % 4 == 0) && aligned16(Input) && aligned16(TransIm) &&
+    // a lane's 4 channels are 16 bytes of fp32 or 8 bytes of bf16
+    const bool vec = (C % 4 == 0) && aligned16(Input) &&
+                     (bf16_out ? (reinterpret_cast<uintptr_t>(TransIm) & 7u) == 0 : aligned16(TransIm)) &&
                      (!AFFINE || (aligned16(Scale) && aligned16(Shift)));
     const bool small = M * C < (1ull << 31);
 #define SWC_DISPATCH(VEC, RELU)                                                                                    \
-    (small ? launch_direct<VEC, RELU, AFFINE, unsigned>(Input, Scale, Shift, TransIm, B, H, W, C, nH, nW, s)       \
-           : launch_direct<VEC, RELU, AFFINE, unsigned long long>(Input, Scale, Shift, TransIm, B, H, W, C, nH, nW, s))
+    (small ? launch_direct<VEC, RELU, AFFINE, unsigned>(Input, Scale, Shift, TransIm, B, H, W, C, nH, nW, bf16_out, s) \
+           : launch_direct<VEC, RELU, AFFINE, unsigned long long>(Input, Scale, Shift, TransIm, B, H, W, C, nH, nW, bf16_out, s))
     if (vec) return relu ? SWC_DISPATCH(4, true) : SWC_DISPATCH(4, false);
     return relu ? SWC_DISPATCH(1, true) : SWC_DISPATCH(1, false);
 #undef SWC_DISPATCH
@@ -223,12 +248,23 @@ int imtrans_entry(const float *Input, const float *Scale, const float *Shift, fl
 extern "C" int swc_winograd2x2_imtrans(const float *Input, float *TransIm, int C, int B, int H, int W,
                                        int pad_h, int pad_w, int relu, swc_stream_t stream)
 {
-    return swc::imtrans_entry<false>(Input, nullptr, nullptr, TransIm, C, B, H, W, pad_h, pad_w, relu, stream);
+    return swc::imtrans_entry<false>(Input, nullptr, nullptr, TransIm, C, B, H, W, pad_h, pad_w, relu, false, stream);
 }
 
 extern "C" int swc_winograd2x2_imtrans_affine(const float *Input, const float *Scale, const float *Shift,
                                               float *TransIm, int C, int B, int H, int W, int pad_h, int pad_w,
                                               int relu, swc_stream_t stream)
 {
-    return swc::imtrans_entry<true>(Input, Scale, Shift, TransIm, C, B, H, W, pad_h, pad_w, relu, stream);
+    return swc::imtrans_entry<true>(Input, Scale, Shift, TransIm, C, B, H, W, pad_h, pad_w, relu, false, stream);
+}
+
+extern "C" int swc_winograd2x2_imtrans_bf16out(const float *Input, const float *Scale, const float *Shift,
+                                               unsigned short *TransIm16, int C, int B, int H, int W, int pad_h,
+                                               int pad_w, int relu, swc_stream_t stream)
+{
+    float *out = reinterpret_cast<float *>(TransIm16);
+    if ((Scale == nullptr) != (Shift == nullptr)) return SWC_ERR_NULL_POINTER;
+    if (Scale != nullptr)
+        return swc::imtrans_entry<true>(Input, Scale, Shift, out, C, B, H, W, pad_h, pad_w, relu, true, stream);
+    return swc::imtrans_entry<false>(Input, nullptr, nullptr, out, C, B, H, W, pad_h, pad_w, relu, true, stream);
 }

@@ -73,6 +73,10 @@ class WinogradUnit(torch.nn.Module):
     def __init__(self, name, c_in, c_out, shortcut, pool, masks, precision, fold_bn=True):
         super().__init__()
         self.name, self.pool, self.fold_bn = name, pool, fold_bn
+        # "bf16": fp32 transformed activations, operands rounded inside the GEMM kernel;
+        # "bf16_stored": the transformed activations themselves are kept in bf16 (needs fold_bn)
+        self.ti_dtype = torch.bfloat16 if precision == "bf16_stored" else torch.float32
+        precision = "bf16" if precision == "bf16_stored" else precision
         self.bn2a = torch.nn.BatchNorm2d(c_in)
         self.conv2a = WinogradConv(c_in, c_out, mask=masks.get("Winograd_W%s_2a/W" % name), precision=precision)
         self.bn2b = torch.nn.BatchNorm2d(c_out)
@@ -89,8 +93,9 @@ class WinogradUnit(torch.nn.Module):
         the Winograd kernels (bn2a, bn2b in the transforms' loads; bn2c and ``+ shortcut`` in the second
         convolution's stores) and the result is already ``shortcut + branch``."""
         if self.fold_bn:
-            h = self.conv2a(WinogradImTrans(_to_nhwc(x), torch.relu, affine=_bn_affine(self.bn2a)))
-            h = self.conv2b(WinogradImTrans(h, torch.relu, affine=_bn_affine(self.bn2b)),
+            dt = self.ti_dtype
+            h = self.conv2a(WinogradImTrans(_to_nhwc(x), torch.relu, affine=_bn_affine(self.bn2a), out_dtype=dt))
+            h = self.conv2b(WinogradImTrans(h, torch.relu, affine=_bn_affine(self.bn2b), out_dtype=dt),
                             affine=_bn_affine(self.bn2c), residual=_to_nhwc(shortcut))
             return _to_nchw(h)
         h = _to_nchw(self.conv2a(WinogradImTrans(_to_nhwc(self.bn2a(x)), torch.relu)))
@@ -111,7 +116,8 @@ class WinogradUnit(torch.nn.Module):
 
 class ResNet18Var(torch.nn.Module):
     """``masks``: optional dict of 0/1 arrays keyed like the reference's pruning masks
-    ('Winograd_W2a_2a/W', ...; prune_script.py:68-78).  ``precision``: 'fp32' or 'bf16' GEMM operands."""
+    ('Winograd_W2a_2a/W', ...; prune_script.py:68-78).  ``precision``: 'fp32' or 'bf16' GEMM operands, or 'bf16_stored' (bf16 operands with
+    the transformed activations also stored as bf16; needs ``fold_bn``)."""
 
     def __init__(self, masks=None, precision="fp32", num_classes=1000, fold_bn=True):
         super().__init__()

@@ -23,6 +23,7 @@ C_SYMBOLS = (
     "swc_strerror", "swc_last_hip_error", "swc_version", "swc_winograd2x2_conv_last_kernel",
     "swc_winograd2x2_imtrans", "swc_winograd2x2_imtrans_affine", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
     "swc_winograd2x2_conv_epilogue",
+    "swc_winograd2x2_imtrans_bf16out", "swc_winograd2x2_weights_bf16", "swc_winograd2x2_conv_bf16in",
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
     "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad", "swc_winograd2x2_relu_conv",
@@ -80,6 +81,12 @@ def lib():
             f.argtypes = [fp, fp, fp, fp, vp] + [i32] * 7 + [vp]
         L.swc_winograd2x2_conv_epilogue.restype = i32
         L.swc_winograd2x2_conv_epilogue.argtypes = [fp] * 6 + [i32] * 8 + [vp]
+        L.swc_winograd2x2_imtrans_bf16out.restype = i32
+        L.swc_winograd2x2_imtrans_bf16out.argtypes = [fp, fp, fp, fp] + [i32] * 7 + [vp]
+        L.swc_winograd2x2_weights_bf16.restype = i32
+        L.swc_winograd2x2_weights_bf16.argtypes = [fp, fp, i32, i32, vp]
+        L.swc_winograd2x2_conv_bf16in.restype = i32
+        L.swc_winograd2x2_conv_bf16in.argtypes = [fp] * 6 + [i32] * 7 + [vp]
         L.swc_winograd2x2_imtrans_op_shape.restype = i32
         L.swc_winograd2x2_imtrans_op_shape.argtypes = [i32, i64p, i64p]
         L.swc_winograd2x2_imtrans_op_compute.restype = i32
@@ -107,16 +114,18 @@ def check(status, where):
         raise SwcError(status, where)
 
 
-def require_cuda_f32(t, name, rank):
-    """The checks a TensorFlow kernel registration did implicitly (float, DEVICE_GPU)."""
+def require_cuda_f32(t, name, rank, dtype=None):
+    """The checks a TensorFlow kernel registration did implicitly (float, DEVICE_GPU).
+    ``dtype`` other than float32 is only used by the bf16-stored variant."""
     import torch
 
+    dtype = torch.float32 if dtype is None else dtype
     if not isinstance(t, torch.Tensor):
         raise TypeError("%s must be a torch.Tensor, got %s" % (name, type(t).__name__))
     if t.dim() != rank:
         raise ValueError("%s must have rank %d, got shape %s" % (name, rank, tuple(t.shape)))
-    if t.dtype != torch.float32:
-        raise TypeError("%s must be float32, got %s" % (name, t.dtype))
+    if t.dtype != dtype:
+        raise TypeError("%s must be %s, got %s" % (name, str(dtype).replace("torch.", ""), t.dtype))
     if not t.is_cuda:
         # The reference's CPU kernels print a message and exit(-1)
         # (winograd2x2_imTrans_op.cc:82-83, winograd2x2_conv_op.cc:89-90); here it is an error.

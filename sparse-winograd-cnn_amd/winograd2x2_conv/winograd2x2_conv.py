@@ -65,6 +65,57 @@ def _forward(I, W, precision, out, scale=None, shift=None, residual=None):
     return out
 
 
+def winograd2x2_weights_bf16(W):
+    """W [16,C,K] float32 -> [16,K,C] bfloat16 (round to nearest even, transposed): the weight layout
+    ``winograd2x2_conv`` reads when its input is a bfloat16 tensor.  Prepare once per weight update."""
+    W = swc_hip.require_cuda_f32(W, "W", 3)
+    if W.shape[0] != 16:
+        raise ValueError("W must have shape [16,C,K]")
+    out = torch.empty((16, W.shape[2], W.shape[1]), dtype=torch.bfloat16, device=W.device)
+    with torch.cuda.device(W.device):
+        st = swc_hip.lib().swc_winograd2x2_weights_bf16(W.data_ptr(), out.data_ptr(), W.shape[1], W.shape[2],
+                                                        torch.cuda.current_stream().cuda_stream)
+    swc_hip.check(st, "winograd2x2_weights_bf16")
+    return out
+
+
+def _forward_bf16_stored(I, W, out, scale, shift, residual):
+    """I [16,B,nH,nW,C] bfloat16; W [16,C,K] float32 or prepared [16,K,C] bfloat16."""
+    I = swc_hip.require_cuda_f32(I, "I", 5, torch.bfloat16)
+    if not isinstance(W, torch.Tensor) or W.dim() != 3:
+        raise ValueError("W must be a rank-3 tensor")
+    if W.dtype == torch.float32:
+        W = winograd2x2_weights_bf16(W)
+    W = swc_hip.require_cuda_f32(W, "W", 3, torch.bfloat16)
+    _, B, nH, nW, C = I.shape
+    if I.shape[0] != 16 or W.shape[0] != 16 or W.shape[2] != C or W.device != I.device:
+        raise ValueError("I must be [16,B,nH,nW,C] and the prepared W [16,K,C] on the same device")
+    K = W.shape[1]
+    shape = (B, 2 * nH, 2 * nW, K)
+    if out is None:
+        out = torch.empty(shape, dtype=torch.float32, device=I.device)
+    elif tuple(out.shape) != shape or out.dtype != torch.float32 or out.device != I.device or not out.is_contiguous():
+        raise ValueError("out must be a contiguous float32 tensor of shape %s on %s" % (shape, I.device))
+    if (scale is None) != (shift is None):
+        raise ValueError("scale and shift go together")
+    if scale is not None:
+        scale = swc_hip.require_cuda_f32(scale, "scale", 1)
+        shift = swc_hip.require_cuda_f32(shift, "shift", 1)
+        if scale.shape[0] != K or shift.shape[0] != K:
+            raise ValueError("scale and shift must have one entry per output channel (%d)" % K)
+    if residual is not None:
+        residual = swc_hip.require_cuda_f32(residual, "residual", 4)
+        if tuple(residual.shape) != shape:
+            raise ValueError("residual must have the output's shape %s" % (shape,))
+    with torch.cuda.device(I.device):
+        st = swc_hip.lib().swc_winograd2x2_conv_bf16in(
+            I.data_ptr(), W.data_ptr(), out.data_ptr(), None if scale is None else scale.data_ptr(),
+            None if shift is None else shift.data_ptr(), None if residual is None else residual.data_ptr(),
+            C, B, nH, nW, K, 1, 1, torch.cuda.current_stream().cuda_stream)
+    swc_hip.check(st, "winograd2x2_conv (bf16-stored operands)")
+    return out
+
+
 def winograd2x2_conv_grad(i1, i2, grad):
     """(I [16,B,nH,nW,C], W [16,C,K], grad [B,2nH,2nW,K]) -> (dI, dW), as the reference's
     winograd2x2_conv_grad (winograd2x2_conv.py:16-17).  fp32 throughout."""
@@ -105,6 +156,9 @@ class _ConvFunction(torch.autograd.Function):
 def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, residual=None):
     """I: [16,B,nH,nW,C], W: [16,C,K], float32 on the GPU -> [B,2nH,2nW,K] (uncropped).
 
+    A bfloat16 ``I`` (from ``winograd2x2_imTrans(..., out_dtype=torch.bfloat16)``) takes the bf16-stored
+    kernel (forward only, needs C % 64 == 0); ``W`` is then float32 [16,C,K] (converted on every call) or the
+    tensor ``winograd2x2_weights_bf16`` prepared from it.
     ``scale``/``shift`` ([K]) and ``residual`` ([B,2nH,2nW,K]), forward only: the result becomes
     ``conv*scale + shift + residual`` inside the kernel's stores (an inference BatchNorm and the
     residual add that follow the second convolution of a ResNet unit).
@@ -113,6 +167,10 @@ def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, r
     through ``winograd2x2_conv_grad`` when an input requires grad.
     """
     needs_grad = torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (I, W))
+    if isinstance(I, torch.Tensor) and I.dtype == torch.bfloat16:
+        if needs_grad:
+            raise NotImplementedError("the bf16-stored variant is forward only")
+        return _forward_bf16_stored(I, W, out, scale, shift, residual)
     if (scale is not None or residual is not None) and needs_grad:
         raise NotImplementedError("the scale/shift/residual epilogue is forward only")
     if out is None and needs_grad:

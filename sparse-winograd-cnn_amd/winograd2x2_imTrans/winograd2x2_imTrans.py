@@ -22,7 +22,7 @@ def winograd2x2_imTrans_shape(shape):
     return tuple(out)
 
 
-def _forward(I, relu, out, scale=None, shift=None):
+def _forward(I, relu, out, scale=None, shift=None, out_dtype=torch.float32):
     I = swc_hip.require_cuda_f32(I, "I", 4)
     shape = winograd2x2_imTrans_shape(I.shape)
     if (scale is None) != (shift is None):
@@ -32,14 +32,21 @@ def _forward(I, relu, out, scale=None, shift=None):
         shift = swc_hip.require_cuda_f32(shift, "shift", 1)
         if scale.shape[0] != I.shape[3] or shift.shape[0] != I.shape[3]:
             raise ValueError("scale and shift must have one entry per channel (%d)" % I.shape[3])
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("out_dtype must be torch.float32 or torch.bfloat16")
     if out is None:
-        out = torch.empty(shape, dtype=torch.float32, device=I.device)
+        out = torch.empty(shape, dtype=out_dtype, device=I.device)
     else:
-        if tuple(out.shape) != shape or out.dtype != torch.float32 or out.device != I.device or not out.is_contiguous():
-            raise ValueError("out must be a contiguous float32 tensor of shape %s on %s" % (shape, I.device))
+        if tuple(out.shape) != shape or out.dtype != out_dtype or out.device != I.device or not out.is_contiguous():
+            raise ValueError("out must be a contiguous %s tensor of shape %s on %s" % (out_dtype, shape, I.device))
     with torch.cuda.device(I.device):
         stream = torch.cuda.current_stream().cuda_stream
-        if scale is not None:
+        if out_dtype == torch.bfloat16:
+            B, H, W, C = I.shape
+            st = swc_hip.lib().swc_winograd2x2_imtrans_bf16out(
+                I.data_ptr(), None if scale is None else scale.data_ptr(), None if shift is None else shift.data_ptr(),
+                out.data_ptr(), C, B, H, W, 1, 1, int(bool(relu)), stream)
+        elif scale is not None:
             B, H, W, C = I.shape
             st = swc_hip.lib().swc_winograd2x2_imtrans_affine(
                 I.data_ptr(), scale.data_ptr(), shift.data_ptr(), out.data_ptr(), C, B, H, W, 1, 1, int(bool(relu)),
@@ -99,11 +106,13 @@ class _ImTransFunction(torch.autograd.Function):
         return winograd2x2_imTrans_grad(grad.contiguous(), ctx.hw[0], ctx.hw[1], relu_output), None
 
 
-def winograd2x2_imTrans(I, relu=False, out=None, scale=None, shift=None):
+def winograd2x2_imTrans(I, relu=False, out=None, scale=None, shift=None, out_dtype=torch.float32):
     """I: [B,H,W,C] float32 NHWC on the GPU -> [16,B,nH,nW,C].
 
     ``scale``/``shift`` ([C] each, forward only): the transform of ``I*scale + shift`` (one fused
     multiply-add per pixel, zero padding left at zero) -- an inference-mode BatchNorm folded into the load.
+    ``out_dtype=torch.bfloat16`` (forward only): the result is rounded to bf16 as it is stored, for
+    ``winograd2x2_conv`` to read back at half the traffic.
 
     ``relu=True`` applies the Winograd-domain ReLU inside the same kernel (what
     ``nl(winograd2x2_imTrans(x))`` with ``nl=tf.nn.relu`` computes in
@@ -111,8 +120,8 @@ def winograd2x2_imTrans(I, relu=False, out=None, scale=None, shift=None):
     Differentiable: gradients flow through ``winograd2x2_imTrans_grad``.
     """
     needs_grad = isinstance(I, torch.Tensor) and I.requires_grad and torch.is_grad_enabled()
-    if scale is not None and needs_grad:
-        raise NotImplementedError("the scale/shift variant is forward only")
+    if (scale is not None or out_dtype != torch.float32) and needs_grad:
+        raise NotImplementedError("the scale/shift and bf16-output variants are forward only")
     if out is None and needs_grad:
         return _ImTransFunction.apply(I, relu)
-    return _forward(I, relu, out, scale, shift)
+    return _forward(I, relu, out, scale, shift, out_dtype)

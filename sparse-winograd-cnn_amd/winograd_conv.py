@@ -46,10 +46,21 @@ class WinogradConv(torch.nn.Module):
             mask = torch.as_tensor(mask, dtype=torch.float32, device=W.device).reshape(W.shape).clone()
         self.register_buffer("mask", mask)
         self._masked = None
+        self._bf16 = None
 
     def refresh(self):
-        """Recompute the cached W*mask (call after changing W or mask)."""
+        """Recompute the cached W*mask and its bf16 copy (call after changing W or mask)."""
         self._masked = None
+        self._bf16 = None
+
+    def bf16_weight(self):
+        """W*mask as the [16,K,C] bfloat16 tensor the bf16-stored kernel reads; cached like masked_weight()."""
+        w = self.masked_weight()
+        cached = getattr(self, "_bf16", None)
+        if cached is None or cached[0] is not w or cached[1] != w._version or cached[2].device != w.device:
+            cached = (w, w._version, winograd2x2_conv.winograd2x2_conv.winograd2x2_weights_bf16(w))
+            self._bf16 = cached
+        return cached[2]
 
     def masked_weight(self):
         if self.mask is None:
@@ -61,7 +72,9 @@ class WinogradConv(torch.nn.Module):
     def forward(self, x, affine=None, residual=None):
         """``affine=(scale, shift)`` and ``residual`` (forward only) are applied to the result inside
         the kernel: ``conv*scale + shift + residual``."""
-        if torch.is_grad_enabled() and self.W.requires_grad:
+        if x.dtype == torch.bfloat16:      # bf16-stored activations: forward only
+            w = self.bf16_weight()
+        elif torch.is_grad_enabled() and self.W.requires_grad:
             w = self.W if self.mask is None else self.W * self.mask
         else:
             w = self.masked_weight()

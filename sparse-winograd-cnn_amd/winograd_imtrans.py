@@ -17,21 +17,22 @@ def identity(x):
 _RELUS = (torch.relu, torch.nn.functional.relu)
 
 
-def WinogradImTrans(x, nl=identity, affine=None):
+def WinogradImTrans(x, nl=identity, affine=None, out_dtype=torch.float32):
     """``nl(winograd2x2_imTrans(x))`` as in the reference (winograd_imtrans.py:16-17).
 
     ``affine=(scale, shift)`` (forward only) transforms ``x*scale + shift`` instead of ``x``: the
     inference-mode BatchNorm that precedes every call in the reference model, folded into the kernel.
+    ``out_dtype=torch.bfloat16`` (forward only) stores the result as bf16 for the bf16-stored convolution.
 
     ``nl`` may be a callable or the strings "identity"/"relu".  A ReLU (``torch.relu``,
     ``torch.nn.functional.relu``, an ``nn.ReLU`` module, or "relu") is fused into the
     transform kernel; any other callable is applied to the op's result.
     """
     op = winograd2x2_imTrans.winograd2x2_imTrans.winograd2x2_imTrans
-    if affine is not None:
-        scale, shift = affine
+    if affine is not None or out_dtype != torch.float32:
+        scale, shift = affine if affine is not None else (None, None)
         base = op
-        op = lambda t, relu=False: base(t, relu=relu, scale=scale, shift=shift)  # noqa: E731
+        op = lambda t, relu=False: base(t, relu=relu, scale=scale, shift=shift, out_dtype=out_dtype)  # noqa: E731
     if nl is None or nl is identity or nl == "identity":
         return op(x)
     if nl == "relu" or isinstance(nl, torch.nn.ReLU) or any(nl is f for f in _RELUS):

@@ -1,0 +1,107 @@
+"""bf16-stored forward pair: imTrans writing bf16, the convolution reading bf16 activations and
+prepared bf16 weights.  Through the C ABI (via the Python mirror), against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import rel_max
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available()
+    import swc_hip
+    swc_hip.lib()
+    return torch.device("cuda:0")
+
+
+def gpu(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def bits(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("shape", [(3, 6, 6, 32), (2, 7, 7, 5), (2, 5, 9, 3), (8, 28, 28, 128)])
+def test_imtrans_bf16_output_is_the_rounded_fp32_transform(oracle, dev, shape, relu):
+    from winograd2x2_imTrans.winograd2x2_imTrans import winograd2x2_imTrans
+    rng = np.random.default_rng(61)
+    x = rng.standard_normal(shape).astype(np.float32)
+    want = oracle.bf16_bits(oracle.imtrans(x, relu=relu))
+    got = winograd2x2_imTrans(gpu(x, dev), relu=relu, out_dtype=torch.bfloat16)
+    assert got.dtype == torch.bfloat16
+    assert np.array_equal(bits(got), want)
+    # with the folded affine map
+    scale = (0.5 + rng.random(shape[3])).astype(np.float32)
+    shift = rng.standard_normal(shape[3]).astype(np.float32)
+    want = oracle.bf16_bits(oracle.imtrans_affine(x, scale, shift, relu=relu))
+    got = winograd2x2_imTrans(gpu(x, dev), relu=relu, scale=gpu(scale, dev), shift=gpu(shift, dev),
+                              out_dtype=torch.bfloat16)
+    assert np.array_equal(bits(got), want)
+
+
+def test_weight_preparation(oracle, dev):
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_weights_bf16
+    rng = np.random.default_rng(62)
+    w = (rng.standard_normal((16, 24, 40)) * 0.05).astype(np.float32)
+    got = winograd2x2_weights_bf16(gpu(w, dev))
+    assert tuple(got.shape) == (16, 40, 24) and got.dtype == torch.bfloat16
+    assert np.array_equal(bits(got), oracle.bf16_bits(w.transpose(0, 2, 1)))
+
+
+@pytest.mark.parametrize("shape", [
+    (3, 3, 3, 64, 32),      # one 64-channel step per position
+    (2, 3, 5, 128, 100),    # ragged rows (M = 30) and columns (K = 100)
+    (8, 14, 14, 128, 128),  # config 3 geometry, reduced batch
+    (4, 7, 7, 256, 72),
+    (1, 1, 1, 64, 4),
+])
+def test_conv_over_bf16_operands(oracle, dev, shape):
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv, winograd2x2_weights_bf16
+    B, nH, nW, C, K = shape
+    rng = np.random.default_rng(63)
+    ti = np.maximum(rng.standard_normal((16, B, nH, nW, C)), 0).astype(np.float32)
+    w = (rng.standard_normal((16, C, K)) * 0.05).astype(np.float32)
+    ti16, w16 = oracle.round_bf16(ti), oracle.round_bf16(w)
+    want = oracle.conv(ti16, w16, acc64=True)          # products of bf16 values are exact in fp32
+    ti_gpu = gpu(ti16, dev).to(torch.bfloat16)         # exact: the values are already bf16
+    got = winograd2x2_conv(ti_gpu, gpu(w, dev)).cpu().numpy()
+    assert got.shape == want.shape
+    assert rel_max(got, want) <= TOL
+    # prepared weights and the epilogue
+    scale = (0.5 + rng.random(K)).astype(np.float32)
+    shift = rng.standard_normal(K).astype(np.float32)
+    res = rng.standard_normal(want.shape).astype(np.float32)
+    got2 = winograd2x2_conv(ti_gpu, winograd2x2_weights_bf16(gpu(w, dev)), scale=gpu(scale, dev), shift=gpu(shift, dev),
+                            residual=gpu(res, dev)).cpu().numpy()
+    assert np.array_equal(got2, oracle.affine(got, scale, shift) + res)
+    # the same values as the kernel that rounds fp32 operands in its registers
+    same = winograd2x2_conv(gpu(ti, dev), gpu(w, dev), precision="bf16").cpu().numpy()
+    assert rel_max(got, same) <= TOL
+
+
+def test_unsupported_channel_count_is_reported(dev):
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv
+    import swc_hip
+    ti = torch.zeros(16, 1, 2, 2, 48, device=dev, dtype=torch.bfloat16)
+    with pytest.raises(swc_hip.SwcError, match="no kernel"):
+        winograd2x2_conv(ti, torch.zeros(16, 48, 8, device=dev))
+
+
+def test_whole_pair_against_fp32_path(oracle, dev):
+    # config 3 in full: the bf16-stored pair against the fp64-accumulated oracle of the unrounded operands
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv
+    from winograd2x2_imTrans.winograd2x2_imTrans import winograd2x2_imTrans
+    rng = np.random.default_rng(64)
+    x = rng.standard_normal((64, 28, 28, 128)).astype(np.float32)
+    w = (rng.standard_normal((16, 128, 128)) * 0.05).astype(np.float32)
+    y = winograd2x2_conv(winograd2x2_imTrans(gpu(x, dev), relu=True, out_dtype=torch.bfloat16), gpu(w, dev)).cpu().numpy()
+    want = oracle.conv(oracle.imtrans(x, relu=True), w, acc64=True)
+    assert rel_max(y, want) <= 1e-2
+    exact = oracle.conv(oracle.round_bf16(oracle.imtrans(x, relu=True)), oracle.round_bf16(w), acc64=True)
+    assert rel_max(y, exact) <= TOL

@@ -214,3 +214,17 @@ def test_affine_is_a_single_rounding_fma(oracle):
     s2, t2 = -s, np.zeros_like(t)
     assert np.array_equal(oracle.affine(x, s2, t2), (-(x.astype(np.float64) * s)).astype(np.float32))
     assert np.array_equal(oracle.imtrans_affine(x, s, t, relu=True), oracle.imtrans(want, relu=True))
+
+
+def test_round_bf16_is_nearest_even(oracle):
+    import torch
+    rng = np.random.default_rng(78)
+    x = (rng.standard_normal(20000) * 10.0 ** rng.integers(-6, 7, 20000)).astype(np.float32)
+    # exact ties: the 16 dropped bits are 0x8000, with the kept bit odd and even
+    ties = np.array([0x3F808000, 0x3F818000, 0xBF808000, 0xBF818000, 0x00008000, 0x7F7E8000], dtype=np.uint32).view(np.float32)
+    x = np.concatenate([x, ties, np.array([0.0, -0.0, 1.0, 3.0e38], dtype=np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()   # torch's CPU conversion rounds to nearest even
+    got = oracle.round_bf16(x)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(oracle.bf16_bits(x), want.view(np.uint32) >> 16)
+    assert np.array_equal(got[-10:-8].view(np.uint32), np.array([0x3F800000, 0x3F820000], dtype=np.uint32))

@@ -29,7 +29,7 @@ def test_same_padding_rule():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("precision,tol", [("fp32", 1e-3), ("bf16", 5e-2)])
+@pytest.mark.parametrize("precision,tol", [("fp32", 1e-3), ("bf16", 5e-2), ("bf16_stored", 5e-2)])
 def test_forward_matches_oracle_path(oracle, precision, tol):
     # Same module, same weights: once on the GPU through the HIP ops, once on the CPU with the two
     # Winograd ops replaced by the oracle.
@@ -49,11 +49,14 @@ def test_forward_matches_oracle_path(oracle, precision, tol):
         bn.bias.data.normal_(0, 0.1)
     image = torch.from_numpy(rng.standard_normal((2, 64, 64, 3)).astype(np.float32))
 
-    def cpu_imtrans(x, nl=None, affine=None):
+    def cpu_imtrans(x, nl=None, affine=None, out_dtype=torch.float32):
         x = x.numpy()
         if affine is not None:
             x = oracle.affine(x, affine[0].detach().numpy(), affine[1].detach().numpy())
-        return torch.from_numpy(oracle.imtrans(x, relu=True))
+        t = oracle.imtrans(x, relu=True)
+        if out_dtype == torch.bfloat16:     # stored rounded; the CPU chain carries the rounded values as fp32
+            t = oracle.round_bf16(t)
+        return torch.from_numpy(t)
 
     def cpu_conv_forward(self, x, affine=None, residual=None):
         y = oracle.conv(x.numpy(), self.masked_weight().numpy(), acc64=True)
