@@ -239,9 +239,9 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
     if (pad_h != 1 || pad_w != 1) return SWC_ERR_BAD_PAD;
     const size_t M = static_cast<size_t>(B) * nH * nW;
     if (M >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
-    using Steps64 = HbCfg<64, 4, 2>;    // two workgroups per CU
-    using Steps128 = HbCfg<128, 3, 1>;  // one workgroup per CU, half as many (longer) steps
-    if (C % Steps64::BK != 0 || !aligned16(Input16) || !aligned16(Weight16t) || static_cast<size_t>(HB_BM) * C >= (1ull << 30))
+    using Deep = HbCfg<64, 4, 2>;   // 4-deep ring, up to two workgroups per CU
+    using Wide = HbCfg<64, 3, 3>;   // 3-deep ring, up to three workgroups per CU
+    if (C % Deep::BK != 0 || !aligned16(Input16) || !aligned16(Weight16t) || static_cast<size_t>(HB_BM) * C >= (1ull << 30))
         return SWC_ERR_UNSUPPORTED;
     const size_t tiles_m = (M + HB_BM - 1) / HB_BM, tiles_n = (static_cast<size_t>(K) + HB_BN - 1) / HB_BN;
     if (tiles_m * tiles_n >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
@@ -250,9 +250,10 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
     ep.shift = Shift;
     ep.residual = Residual;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // With at most one workgroup per CU anyway, the 128-channel steps measured 17-19 % faster
-    // (ResNet-18 conv4 shapes); with more workgroups than CUs two resident ones per CU win.
-    if (C % Steps128::BK == 0 && tiles_m * tiles_n <= kCUs)
-        return launch_bf16_stored<Steps128>(Input16, Weight16t, Output, M, C, K, nH, nW, tiles_m, tiles_n, ep, s);
-    return launch_bf16_stored<Steps64>(Input16, Weight16t, Output, M, C, K, nH, nW, tiles_m, tiles_n, ep, s);
+    // More resident workgroups hide more of each other's waits once there are enough of them to go round
+    // (conv3: 18.7 vs 19.6 us); a grid that leaves CUs with one workgroup does better with the deeper
+    // ring (conv4b: 30.8 vs 34.2 us).
+    if (tiles_m * tiles_n > kCUs)
+        return launch_bf16_stored<Wide>(Input16, Weight16t, Output, M, C, K, nH, nW, tiles_m, tiles_n, ep, s);
+    return launch_bf16_stored<Deep>(Input16, Weight16t, Output, M, C, K, nH, nW, tiles_m, tiles_n, ep, s);
 }

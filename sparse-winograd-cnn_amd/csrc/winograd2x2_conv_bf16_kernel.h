@@ -125,39 +125,67 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
         a_off[h] = ra * ROW_BYTES + (((2 * h + lg) ^ (ra % CH)) * 16u);
         b_off[h] = Cfg::TILE_BYTES + rb * ROW_BYTES + (((2 * h + lg) ^ (rb % CH)) * 16u);
     }
-    unsigned st_cur = 0;
+    unsigned st_next = 0;  // byte offset of the ring slot whose operands are fetched next
+
+    // The operands of a step are read from LDS one step ahead of the MFMAs that consume them, so that
+    // the matrix work of step s runs while the reads of step s+1 (and the wait for its tiles) are in
+    // flight: two register sets, F[s & 1].
+    bf16x8 fa[2][Cfg::NMFMA], fb[2][Cfg::NMFMA];
+    auto fetch = [&](int set) __attribute__((always_inline)) {
+        // The tiles of the step to fetch have landed once at most the copies of the NSTAGE-2 steps
+        // issued after it are outstanding; after the barrier every wave has also finished reading the
+        // slot that the next copies overwrite (it was fetched one step earlier still).
+        if (!(ABL & 2)) wait_vmcnt<(NSTAGE - 2) * Cfg::COPIES>();
+        if (!(ABL & 1)) __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (!(ABL & 4)) issue();
+#pragma unroll
+        for (int h = 0; h < Cfg::NMFMA; ++h) {
+            if (ABL & 8) {
+                fa[set][h] = bf16x8{};
+                fb[set][h] = bf16x8{};
+                asm volatile("" : "+v"(fa[set][h]), "+v"(fb[set][h]));
+            } else {
+                fa[set][h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_next + a_off[h]);
+                fb[set][h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_next + b_off[h]);
+            }
+        }
+        st_next = st_next + Cfg::STAGE_BYTES == Cfg::LDS_BYTES ? 0 : st_next + Cfg::STAGE_BYTES;
+    };
+    fetch(0);
 
     static_for<16>([&](auto pos_tag) {
         constexpr int pos = decltype(pos_tag)::value;
         floatx16 P = {};
-        for (int kc = 0; kc < nkc; ++kc) {
-            // Step's tiles have landed once at most the copies of the NSTAGE-2 steps after it are
-            // outstanding; after the barrier everyone is also done with the slot the next copies overwrite.
-            if (!(ABL & 2)) wait_vmcnt<(NSTAGE - 2) * Cfg::COPIES>();
-            if (!(ABL & 1)) __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-            if (!(ABL & 4)) issue();
-            bf16x8 a[Cfg::NMFMA], b[Cfg::NMFMA];
+        auto mfmas = [&](int set) __attribute__((always_inline)) {
 #pragma unroll
             for (int h = 0; h < Cfg::NMFMA; ++h) {
-                if (ABL & 8) {
-                    a[h] = bf16x8{};
-                    b[h] = bf16x8{};
-                    asm volatile("" : "+v"(a[h]), "+v"(b[h]));
-                } else {
-                    a[h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_cur + a_off[h]);
-                    b[h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_cur + b_off[h]);
-                }
+                if (ABL & 16)
+                    P[h] += static_cast<float>(fa[set][h][0]) + static_cast<float>(fb[set][h][0]);
+                else
+                    P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][h], fb[set][h], P, 0, 0, 0);
             }
+        };
+        // A position starts with its first step's operands in set 0.  Steps go in pairs so that the set
+        // indices are compile-time constants (the sets must stay in registers); an odd last step moves
+        // the prefetched set 1 into set 0.  Past the very last step the fetch reads the wrapped-around
+        // copy, which is never used.
+        int kc = 0;
+#pragma nounroll
+        for (; kc + 1 < nkc; kc += 2) {
+            fetch(1);
+            mfmas(0);
+            fetch(0);
+            mfmas(1);
+        }
+        if (kc < nkc) {
+            fetch(1);
+            mfmas(0);
 #pragma unroll
             for (int h = 0; h < Cfg::NMFMA; ++h) {
-                if (ABL & 16) {
-                    P[h] += static_cast<float>(a[h][0]) + static_cast<float>(b[h][0]);
-                } else {
-                    P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[h], b[h], P, 0, 0, 0);
-                }
+                fa[0][h] = fa[1][h];
+                fb[0][h] = fb[1][h];
             }
-            st_cur = st_cur + Cfg::STAGE_BYTES == Cfg::LDS_BYTES ? 0 : st_cur + Cfg::STAGE_BYTES;
         }
         // fold P_pos into the running output tiles, ascending pos (winograd2x2_conv_cuda.cu.cc:39-46)
         constexpr unsigned long long plus = kPlus, minus = kMinus;
@@ -167,6 +195,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
                 Y[j][0][0] += P;
             else if ((minus >> (4 * pos + j)) & 1ull)
                 Y[j][0][0] -= P;
+            // pins the update here: otherwise the compiler defers all the adds to the end and keeps the
+            // 16 product tiles alive instead of the 4 sums
+            asm volatile("" : "+v"(Y[j][0][0]));
         }
     });
     wait_vmcnt<0>();  // the surplus copies must land before the workgroup's LDS is handed on
