@@ -465,3 +465,22 @@ def test_host_threads_on_their_own_streams(oracle, dev):
     assert not errors, errors
     for got, want in zip(gots, wants):
         assert rel_max(got, want) <= TOL
+
+
+def test_imtrans_beyond_2_pow_31_elements_per_plane(dev):
+    # M*C >= 2^31 switches the kernel to 64-bit lane indices.  The 137 GB result cannot be checked on the
+    # host; sampled images must equal what the same op returns for them alone (32-bit path).
+    imtrans, _ = ops()
+    free, _total = torch.cuda.mem_get_info(dev)
+    if free < 190e9:
+        pytest.skip("needs 172 GB of free device memory")
+    B, H, W, C = 21500, 56, 56, 128
+    assert B * 28 * 28 * C >= 2 ** 31
+    x = torch.empty(B, H, W, C, device=dev)
+    for i in range(0, B, 500):
+        x[i:i + 500].normal_()
+    ti = imtrans(x, relu=True)
+    for b in (0, 1, 7777, 13699, 13700, B - 1):   # 13699/13700 straddle the 2^31 boundary
+        assert torch.equal(ti[:, b:b + 1], imtrans(x[b:b + 1].contiguous(), relu=True)), b
+    del ti, x
+    torch.cuda.empty_cache()
