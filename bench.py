@@ -113,7 +113,7 @@ def cpu_baseline(name, x, w, budget_s):
 
 
 def bench_resnet(args, torch, dev):
-    """BASELINE config 5: full ResNet-18-var forward, all 16 3x3 convs through the ops, random-init weights
+    """benchmark config 5: full ResNet-18-var forward, all 16 3x3 convs through the ops, random-init weights
     magnitude-pruned per layer (30/20/10/10 % density by stage), input ~N(0,1) [N,224,224,3]."""
     import numpy as np
 

@@ -25,7 +25,7 @@ def gpu(a, dev):
 SHAPES = [
     # B, H, W, C, K
     (3, 6, 6, 32, 32),      # the reference tests' shape
-    (1, 16, 16, 64, 64),    # BASELINE config 1
+    (1, 16, 16, 64, 64),    # benchmark config 1
     (2, 7, 7, 8, 12),       # odd extent, one channel chunk, K below a tile
     (2, 5, 9, 24, 100),     # H != W, ragged K
     (1, 2, 2, 8, 4),        # a single tile

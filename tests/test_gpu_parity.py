@@ -43,7 +43,7 @@ def gpu(a, dev):
 IMTRANS_SHAPES = [
     (3, 6, 6, 32),      # winograd2x2_imTrans_test.py:160-164
     (2, 7, 7, 5),       # odd extent; C % 4 != 0 takes the scalar path
-    (1, 16, 16, 64),    # BASELINE config 1
+    (1, 16, 16, 64),    # benchmark config 1
     (2, 5, 9, 3),
     (1, 1, 1, 1),
     (1, 2, 3, 7),
@@ -88,7 +88,7 @@ CONV_SHAPES = [
     # B, nH, nW, C, K
     (3, 3, 3, 32, 32),     # winograd2x2_conv_test.py:158-162
     (2, 4, 4, 5, 7),       # C=5, K=7 as in winograd2x2_conv_grad_test.py:160-163 (scalar-load path)
-    (1, 8, 8, 64, 64),     # BASELINE config 1
+    (1, 8, 8, 64, 64),     # benchmark config 1
     (1, 1, 1, 1, 1),
     (2, 3, 5, 36, 100),    # ragged in M, C and K tiles
     (2, 14, 14, 64, 128),  # C != K as in Winograd_W3a_2a
@@ -160,7 +160,7 @@ def test_conv_fp32_exact_on_integers(oracle, dev, shape):
 
 
 def test_conv_full_config3(oracle, dev):
-    # BASELINE config 3 at full size: N=64, 28x28x128 -> 128, Winograd-domain ReLU on,
+    # benchmark config 3 at full size: N=64, 28x28x128 -> 128, Winograd-domain ReLU on,
     # weights pruned to 20 % density.
     imtrans, conv = ops()
     rng = np.random.default_rng(300)
@@ -222,7 +222,7 @@ def test_conv_bf16_variant(oracle, dev, shape):
 
 
 def test_full_size_properties(dev):
-    # Size-independent checks at BASELINE config 2 in full (N=64, 56x56x64 -> 64).
+    # Size-independent checks at benchmark config 2 in full (N=64, 56x56x64 -> 64).
     imtrans, conv = ops()
     g = torch.Generator(device="cpu").manual_seed(200)
     x = torch.randn(64, 56, 56, 64, generator=g).clamp_(min=0).to(dev)

@@ -16,7 +16,7 @@ from helpers import (direct_conv, imtrans_matrix, kernel_matrix, output_matrix, 
 SHAPES = [
     (3, 6, 6, 32),    # the reference tests' own shape (winograd2x2_imTrans_test.py:160-164)
     (2, 7, 7, 5),     # odd extent, C not a multiple of 4 (C=5 as in winograd2x2_conv_grad_test.py:160-163)
-    (1, 16, 16, 64),  # BASELINE config 1
+    (1, 16, 16, 64),  # benchmark config 1
     (2, 5, 9, 3),     # H != W, both odd
     (1, 1, 1, 1),     # a single pixel: one tile, mostly padding
     (1, 2, 3, 7),
@@ -151,7 +151,7 @@ def test_kernel_transform_matches_GgGt(oracle):
 @pytest.mark.parametrize("B,H,W,C,K", [
     (3, 6, 6, 32, 32),   # winograd2x2_conv_test.py:158-162
     (2, 7, 7, 5, 7),     # odd size: crop [:, :H, :W] (winograd2x2_conv_test.py:152-153); C != K
-    (1, 16, 16, 64, 64),  # BASELINE config 1
+    (1, 16, 16, 64, 64),  # benchmark config 1
     (2, 5, 8, 3, 9),
 ])
 def test_whole_path_equals_conv2d(oracle, B, H, W, C, K):

@@ -1,4 +1,4 @@
-"""The ResNet-18-var forward harness (BASELINE config 5 topology) with its 16 convs through the ops."""
+"""The ResNet-18-var forward harness (benchmark config 5 topology) with its 16 convs through the ops."""
 import numpy as np
 import pytest
 import torch
