@@ -264,11 +264,18 @@ def main():
         f_imtrans()
         f_conv()
 
-    fused_ok = args.precision == "fp32" and L.swc_winograd2x2_relu_conv(xp, wp, yp, C, B, H, W, K, 1, 1, 1, stream) == 0
+    # the same layer as one kernel: fp32 (swc_winograd2x2_relu_conv) or bf16 operands (swc_winograd2x2_relu_conv_bf16)
+    def call_fused():
+        if stored:
+            return L.swc_winograd2x2_relu_conv_bf16(xp, None, None, w16p, yp, None, None, None, C, B, H, W, K, 1, 1, 1,
+                                                    stream)
+        return L.swc_winograd2x2_relu_conv(xp, wp, yp, C, B, H, W, K, 1, 1, 1, stream)
+
+    fused_ok = args.precision != "bf16" and call_fused() == 0
 
     def f_fused():
-        if L.swc_winograd2x2_relu_conv(xp, wp, yp, C, B, H, W, K, 1, 1, 1, stream) != 0:
-            raise RuntimeError("swc_winograd2x2_relu_conv failed")
+        if call_fused() != 0:
+            raise RuntimeError("the fused-layer launcher failed")
 
     for _ in range(args.warmup):
         step()
@@ -411,8 +418,11 @@ def main():
             "ms": round(ms_fused, 5),
             "effective_direct_conv_GFLOPs": round(direct_flops / (ms_fused * 1e-3) / 1e9, 1),
             "mfma_TFLOPs": round(gemm_flops / (ms_fused * 1e-3) / 1e12, 2),
-            "mfma_frac": round(gemm_flops / (ms_fused * 1e-3) / 1e12 / FP32_MFMA_PEAK_TF, 4),
-            "algorithmic_bytes_per_launch": 4.0 * B * H * W * C + 64.0 * C * K + 16.0 * M * K,
+            "mfma_frac": round(gemm_flops / (ms_fused * 1e-3) / 1e12 /
+                               (BF16_MFMA_PEAK_TF if stored else FP32_MFMA_PEAK_TF), 4),
+            "algorithmic_bytes_per_launch": 4.0 * B * H * W * C + 16.0 * (2.0 if stored else 4.0) * C * K + 16.0 * M * K,
+            "hbm_frac": round((4.0 * B * H * W * C + 16.0 * (2.0 if stored else 4.0) * C * K + 16.0 * M * K) /
+                              (ms_fused * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "max_abs_diff_vs_two_op": float((y_fused - y).abs().max()),
         },
         "roofline_imtrans": {

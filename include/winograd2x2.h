@@ -212,6 +212,18 @@ SWC_API int swc_winograd2x2_conv_bf16in(const uint16_t *Input16, const uint16_t 
                                 const float *Scale, const float *Shift, const float *Residual, int C, int B,
                                 int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream);
 
+/* The whole layer in one kernel with bf16 GEMM operands: the values of swc_winograd2x2_imtrans_bf16out
+ * (with InScale/InShift as in swc_winograd2x2_imtrans_affine, or NULL) followed by
+ * swc_winograd2x2_conv_bf16in (with OutScale/OutShift/Residual as in swc_winograd2x2_conv_epilogue, or
+ * NULL), without the transformed activations ever reaching memory.
+ *   Input [B,H,W,C] fp32, Weight16t [16,K,C] bf16 (swc_winograd2x2_weights_bf16)  ->  Output [B,2nH,2nW,K] fp32
+ * No counterpart in the reference.  Needs C % 16 == 0 and 16-byte aligned operands; returns
+ * SWC_ERR_UNSUPPORTED otherwise (use the two entry points above). */
+SWC_API int swc_winograd2x2_relu_conv_bf16(const float *Input, const float *InScale, const float *InShift,
+                                   const uint16_t *Weight16t, float *Output, const float *OutScale,
+                                   const float *OutShift, const float *Residual, int C, int B, int H, int W,
+                                   int K, int pad_h, int pad_w, int relu, swc_stream_t stream);
+
 /* ---------------------------------------------------------------------------
  * Backward ops.
  * ------------------------------------------------------------------------- */

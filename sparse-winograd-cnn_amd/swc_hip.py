@@ -24,6 +24,7 @@ C_SYMBOLS = (
     "swc_winograd2x2_imtrans", "swc_winograd2x2_imtrans_affine", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
     "swc_winograd2x2_conv_epilogue",
     "swc_winograd2x2_imtrans_bf16out", "swc_winograd2x2_weights_bf16", "swc_winograd2x2_conv_bf16in",
+    "swc_winograd2x2_relu_conv_bf16",
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
     "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad", "swc_winograd2x2_relu_conv",
@@ -87,6 +88,8 @@ def lib():
         L.swc_winograd2x2_weights_bf16.argtypes = [fp, fp, i32, i32, vp]
         L.swc_winograd2x2_conv_bf16in.restype = i32
         L.swc_winograd2x2_conv_bf16in.argtypes = [fp] * 6 + [i32] * 7 + [vp]
+        L.swc_winograd2x2_relu_conv_bf16.restype = i32
+        L.swc_winograd2x2_relu_conv_bf16.argtypes = [fp] * 8 + [i32] * 8 + [vp]
         L.swc_winograd2x2_imtrans_op_shape.restype = i32
         L.swc_winograd2x2_imtrans_op_shape.argtypes = [i32, i64p, i64p]
         L.swc_winograd2x2_imtrans_op_compute.restype = i32

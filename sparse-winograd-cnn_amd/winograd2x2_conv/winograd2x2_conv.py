@@ -207,3 +207,63 @@ def winograd2x2_relu_conv(X, W, relu=True, out=None):
         return _forward(_it.winograd2x2_imTrans(X, relu=relu), W, "fp32", out)
     swc_hip.check(st, "winograd2x2_relu_conv")
     return out
+
+
+def winograd2x2_relu_conv_bf16(X, W, relu=True, out=None, in_affine=None, scale=None, shift=None, residual=None):
+    """The layer pair in one kernel with bf16 GEMM operands: the values of
+    ``winograd2x2_conv(winograd2x2_imTrans(X, relu, out_dtype=bfloat16), W16)``, the transformed
+    activations never reaching memory.
+
+    X: [B,H,W,C] float32 NHWC; W: float32 [16,C,K] (converted on every call) or the bfloat16 [16,K,C]
+    tensor from ``winograd2x2_weights_bf16``.  ``in_affine=(scale, shift)`` ([C] each) maps the input as
+    ``winograd2x2_imTrans(..., scale, shift)`` does; ``scale``/``shift`` ([K]) and ``residual`` act on the
+    result as in ``winograd2x2_conv``.  Shapes the kernel does not cover (C % 16 != 0, ...) run the
+    bf16-stored pair, or the fp32-stored pair with bf16 operands, instead.  Forward only.
+    """
+    import winograd2x2_imTrans.winograd2x2_imTrans as _it
+
+    X = swc_hip.require_cuda_f32(X, "X", 4)
+    W_in = W
+    if isinstance(W, torch.Tensor) and W.dtype == torch.float32:
+        W = winograd2x2_weights_bf16(W)
+    W = swc_hip.require_cuda_f32(W, "W", 3, torch.bfloat16)
+    B, H, Wd, C = X.shape
+    if W.shape[0] != 16 or W.shape[2] != C or W.device != X.device:
+        raise ValueError("the prepared W must have shape [16,K,%d] on X's device, got %s" % (C, tuple(W.shape)))
+    K = W.shape[1]
+    shape = (B, 2 * ((H + 1) // 2), 2 * ((Wd + 1) // 2), K)
+    if out is None:
+        out = torch.empty(shape, dtype=torch.float32, device=X.device)
+    elif tuple(out.shape) != shape or out.dtype != torch.float32 or out.device != X.device or not out.is_contiguous():
+        raise ValueError("out must be a contiguous float32 tensor of shape %s on %s" % (shape, X.device))
+    in_scale, in_shift = in_affine if in_affine is not None else (None, None)
+    if (scale is None) != (shift is None) or (in_scale is None) != (in_shift is None):
+        raise ValueError("scale and shift go together")
+    checked = {}
+    for name, t, n in (("in_scale", in_scale, C), ("in_shift", in_shift, C), ("scale", scale, K), ("shift", shift, K)):
+        if t is not None:
+            t = swc_hip.require_cuda_f32(t, name, 1)
+            if t.shape[0] != n:
+                raise ValueError("%s must have %d entries" % (name, n))
+        checked[name] = t
+    if residual is not None:
+        residual = swc_hip.require_cuda_f32(residual, "residual", 4)
+        if tuple(residual.shape) != shape:
+            raise ValueError("residual must have the output's shape %s" % (shape,))
+    ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
+    with torch.cuda.device(X.device):
+        st = swc_hip.lib().swc_winograd2x2_relu_conv_bf16(
+            X.data_ptr(), ptr(checked["in_scale"]), ptr(checked["in_shift"]), W.data_ptr(), out.data_ptr(),
+            ptr(checked["scale"]), ptr(checked["shift"]), ptr(residual), C, B, H, Wd, K, 1, 1, int(bool(relu)),
+            torch.cuda.current_stream().cuda_stream)
+    if st == swc_hip.SWC_ERR_UNSUPPORTED:
+        if C % 64 == 0:
+            ti = _it.winograd2x2_imTrans(X, relu=relu, scale=checked["in_scale"], shift=checked["in_shift"],
+                                         out_dtype=torch.bfloat16)
+            return _forward_bf16_stored(ti, W, out, checked["scale"], checked["shift"], residual)
+        if W_in.dtype != torch.float32:
+            raise ValueError("this shape needs the float32 weights [16,C,K] (no bf16 kernel takes C = %d)" % C)
+        ti = _it.winograd2x2_imTrans(X, relu=relu, scale=checked["in_scale"], shift=checked["in_shift"])
+        return _forward(ti, W_in, "bf16", out, checked["scale"], checked["shift"], residual)
+    swc_hip.check(st, "winograd2x2_relu_conv_bf16")
+    return out

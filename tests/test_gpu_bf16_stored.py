@@ -105,3 +105,50 @@ def test_whole_pair_against_fp32_path(oracle, dev):
     assert rel_max(y, want) <= 1e-2
     exact = oracle.conv(oracle.round_bf16(oracle.imtrans(x, relu=True)), oracle.round_bf16(w), acc64=True)
     assert rel_max(y, exact) <= TOL
+
+
+@pytest.mark.parametrize("shape", [
+    (3, 6, 6, 16, 32),      # one 16-channel chunk
+    (2, 7, 9, 32, 100),     # odd extent, ragged rows and columns, two chunks
+    (2, 5, 5, 48, 20),      # three chunks (odd count)
+    (8, 28, 28, 128, 128),  # config 3 geometry, reduced batch
+    (4, 14, 14, 256, 72),
+    (1, 2, 2, 64, 4),
+])
+@pytest.mark.parametrize("relu", [True, False])
+def test_fused_bf16_layer(oracle, dev, shape, relu):
+    # One kernel from the fp32 input to the fp32 output must give what the bf16-stored pair gives.
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_relu_conv_bf16, winograd2x2_weights_bf16
+    B, H, W, C, K = shape
+    rng = np.random.default_rng(65)
+    x = rng.standard_normal((B, H, W, C)).astype(np.float32)
+    w = (rng.standard_normal((16, C, K)) * 0.05).astype(np.float32)
+    ti16 = oracle.round_bf16(oracle.imtrans(x, relu=relu))
+    want = oracle.conv(ti16, oracle.round_bf16(w), acc64=True)
+    got = winograd2x2_relu_conv_bf16(gpu(x, dev), gpu(w, dev), relu=relu).cpu().numpy()
+    assert got.shape == want.shape
+    assert rel_max(got, want) <= TOL
+    # folded input affine map and output epilogue, prepared weights
+    s_in = (0.5 + rng.random(C)).astype(np.float32)
+    t_in = rng.standard_normal(C).astype(np.float32)
+    s_out = (0.5 + rng.random(K)).astype(np.float32)
+    t_out = rng.standard_normal(K).astype(np.float32)
+    res = rng.standard_normal(want.shape).astype(np.float32)
+    ti16 = oracle.round_bf16(oracle.imtrans_affine(x, s_in, t_in, relu=relu))
+    core = oracle.conv(ti16, oracle.round_bf16(w), acc64=True)
+    want2 = core.astype(np.float64) * s_out + t_out + res
+    got2 = winograd2x2_relu_conv_bf16(gpu(x, dev), winograd2x2_weights_bf16(gpu(w, dev)), relu=relu,
+                                      in_affine=(gpu(s_in, dev), gpu(t_in, dev)), scale=gpu(s_out, dev),
+                                      shift=gpu(t_out, dev), residual=gpu(res, dev)).cpu().numpy()
+    assert rel_max(got2, want2) <= TOL
+
+
+def test_fused_bf16_layer_falls_back(oracle, dev):
+    # C = 40 is no multiple of 16: the wrapper runs the fp32-stored pair with bf16 operands (still HIP).
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_relu_conv_bf16
+    rng = np.random.default_rng(66)
+    x = rng.standard_normal((2, 6, 6, 40)).astype(np.float32)
+    w = (rng.standard_normal((16, 40, 12)) * 0.05).astype(np.float32)
+    want = oracle.conv(oracle.round_bf16(oracle.imtrans(x, relu=True)), oracle.round_bf16(w), acc64=True)
+    got = winograd2x2_relu_conv_bf16(gpu(x, dev), gpu(w, dev)).cpu().numpy()
+    assert rel_max(got, want) <= TOL
