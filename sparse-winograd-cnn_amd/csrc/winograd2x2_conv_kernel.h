@@ -627,8 +627,8 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
 
     // ---- main loop ----------------------------------------------------------------------------
     // A wave issues at most one instruction every four cycles and an MFMA occupies the matrix
-    // pipe for 64, so everything that is not an MFMA is dealt out between the MFMAs, a few
-    // instructions after each (sched_barrier pins the order):
+    // pipe for 64 (32x32x2) or 32 (16x16x4) cycles, so everything that is not an MFMA is dealt out
+    // between the MFMAs, a few instructions after each (sched_barrier pins the order):
     //   first half  (MFMAs on F1): the LDS reads of the step's second half F2;
     //   second half (MFMAs on F2): after the first MFMA, wait for the tile of step s+1 and
     //     barrier (everyone now holds step s entirely in registers, so its ring slot is free);
