@@ -81,23 +81,44 @@ __global__ __launch_bounds__(256) void output_transform_grad_kernel(const float 
 // and the same combination over v for the column, the own tile needs all 16 planes once, each edge
 // neighbour one row or column of 4 planes and each corner one plane: 36 loads for 4 pixels where the
 // per-pixel form issues 64.
+// A workgroup takes a block of IG_TILES tiles of one image, rh rows by rw = 1 << rw_shift columns,
+// and IG_LANES channel vectors of each.  Every lane loads its own tile's 16 planes once and leaves in
+// LDS the 12 sums its neighbours need of them (two per edge, one per corner); a neighbour inside the
+// block is read from there, one outside it from memory as above.  With every neighbour read from
+// memory the kernel fetched 1.9 times the planes' size: the planes in flight exceed the L2 by far,
+// so a second reader rarely hits.
+constexpr int IG_LANES = 8;    // channel vectors per tile in a workgroup (128 contiguous bytes at VEC 4)
+constexpr int IG_THREADS = 256;
+constexpr int IG_TILES = IG_THREADS / IG_LANES;
+// slots of the exchange: what a tile offers to the tile below, above, to the right, to the left
+// (two sums each) and to its four diagonal neighbours
+enum { IG_TO_BELOW = 0, IG_TO_ABOVE = 2, IG_TO_RIGHT = 4, IG_TO_LEFT = 6, IG_C33 = 8, IG_C30 = 9, IG_C03 = 10, IG_C00 = 11, IG_SLOTS = 12 };
+
+// grid.x = cgroups * blocks_x * blocks_y * B
 template <int VEC, bool MASK>
-__global__ __launch_bounds__(256) void imtrans_grad_tile_kernel(const float *__restrict__ dT,
-                                                                const float *__restrict__ mask_src,
-                                                                float *__restrict__ dX, int H, int W, int C, int nH,
-                                                                int nW, unsigned items, size_t plane)
+__global__ __launch_bounds__(IG_THREADS) void imtrans_grad_tile_kernel(const float *__restrict__ dT,
+                                                                       const float *__restrict__ mask_src,
+                                                                       float *__restrict__ dX, int H, int W, int C, int nH,
+                                                                       int nW, unsigned cgroups, unsigned blocks_x,
+                                                                       unsigned blocks_y, int rw_shift, size_t plane)
 {
     using V = typename GVec<VEC>::type;
-    const unsigned idx = xcd_swizzle(blockIdx.x, gridDim.x) * 256 + threadIdx.x;
-    if (idx >= items) return;
+    __shared__ V ex[IG_SLOTS][IG_THREADS];
+    // consecutive logical ids are the channel groups of one block of tiles
+    unsigned id = xcd_swizzle(blockIdx.x, gridDim.x);
+    const unsigned cgroup = id % cgroups;
+    id /= cgroups;
+    const unsigned bxi = id % blocks_x;
+    id /= blocks_x;
+    const unsigned byi = id % blocks_y, b = id / blocks_y;
     const unsigned CV = C / VEC;
-    const unsigned cv = idx % CV;
-    unsigned m = idx / CV;
-    const int tw = m % nW;
-    m /= nW;
-    const int th = m % nH;
-    const unsigned b = m / nH;
-    // masked gradient of plane 4u+v at tile (th+dy, tw+dx), zero outside the tile grid
+    const unsigned cv = cgroup * IG_LANES + threadIdx.x % IG_LANES;
+    const int tl = threadIdx.x / IG_LANES;            // tile within the block
+    const int rw = 1 << rw_shift, rh = IG_TILES >> rw_shift;
+    const int ty = tl >> rw_shift, tx = tl & (rw - 1);
+    const int th = static_cast<int>(byi) * rh + ty, tw = static_cast<int>(bxi) * rw + tx;
+    const bool valid = th < nH && tw < nW && cv < CV;
+    // masked gradient of plane 4u+v at tile (th+dy, tw+dx)
     auto g = [&](int u, int v, int dy, int dx) __attribute__((always_inline)) -> V {
         const size_t off = static_cast<size_t>(4 * u + v) * plane +
                            ((static_cast<size_t>(b) * nH + (th + dy)) * nW + (tw + dx)) * C + static_cast<size_t>(cv) * VEC;
@@ -115,46 +136,101 @@ __global__ __launch_bounds__(256) void imtrans_grad_tile_kernel(const float *__r
     auto mid = [](int a, V e0, V e1, V e2, V e3) __attribute__((always_inline)) -> V {
         return a == 0 ? add(sub(e1, e2), e3) : add(sub(e1, e0), e2);
     };
-    const bool up = th > 0, down = th + 1 < nH, left = tw > 0, right = tw + 1 < nW;
     V out[2][2];
-    {   // own tile: rows 1+a, then columns 1+b
+    if (valid) {   // own tile: rows 1+a, then columns 1+b; and what the neighbours need of it
+        V t[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) t[u][v] = g(u, v, 0, 0);
         V row[2][4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            const V e0 = g(0, v, 0, 0), e1 = g(1, v, 0, 0), e2 = g(2, v, 0, 0), e3 = g(3, v, 0, 0);
-            row[0][v] = mid(0, e0, e1, e2, e3);
-            row[1][v] = mid(1, e0, e1, e2, e3);
+            row[0][v] = mid(0, t[0][v], t[1][v], t[2][v], t[3][v]);
+            row[1][v] = mid(1, t[0][v], t[1][v], t[2][v], t[3][v]);
         }
 #pragma unroll
         for (int a = 0; a < 2; ++a)
 #pragma unroll
             for (int bb = 0; bb < 2; ++bb) out[a][bb] = mid(bb, row[a][0], row[a][1], row[a][2], row[a][3]);
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            ex[IG_TO_BELOW + q][threadIdx.x] = mid(q, t[3][0], t[3][1], t[3][2], t[3][3]);
+            ex[IG_TO_ABOVE + q][threadIdx.x] = mid(q, t[0][0], t[0][1], t[0][2], t[0][3]);
+            ex[IG_TO_RIGHT + q][threadIdx.x] = mid(q, t[0][3], t[1][3], t[2][3], t[3][3]);
+            ex[IG_TO_LEFT + q][threadIdx.x] = mid(q, t[0][0], t[1][0], t[2][0], t[3][0]);
+        }
+        ex[IG_C33][threadIdx.x] = t[3][3];
+        ex[IG_C30][threadIdx.x] = t[3][0];
+        ex[IG_C03][threadIdx.x] = t[0][3];
+        ex[IG_C00][threadIdx.x] = t[0][0];
     }
+    __syncthreads();
+    if (!valid) return;
+
+    const bool up = th > 0, down = th + 1 < nH, left = tw > 0, right = tw + 1 < nW;
+    // the neighbour at (dy, dx) is lane threadIdx.x + nb(dy, dx) of this workgroup if its tile is in the block
+    auto nb = [&](int dy, int dx) __attribute__((always_inline)) { return (dy * rw + dx) * IG_LANES; };
+    auto inside = [&](int dy, int dx) __attribute__((always_inline)) {
+        return ty + dy >= 0 && ty + dy < rh && tx + dx >= 0 && tx + dx < rw;
+    };
     if (up) {      // row 3 of the tile above: -dT[3][v]
-        const V e0 = g(3, 0, -1, 0), e1 = g(3, 1, -1, 0), e2 = g(3, 2, -1, 0), e3 = g(3, 3, -1, 0);
-        out[0][0] = sub(out[0][0], mid(0, e0, e1, e2, e3));
-        out[0][1] = sub(out[0][1], mid(1, e0, e1, e2, e3));
+        V s0, s1;
+        if (inside(-1, 0)) {
+            s0 = ex[IG_TO_BELOW][threadIdx.x + nb(-1, 0)];
+            s1 = ex[IG_TO_BELOW + 1][threadIdx.x + nb(-1, 0)];
+        } else {
+            const V e0 = g(3, 0, -1, 0), e1 = g(3, 1, -1, 0), e2 = g(3, 2, -1, 0), e3 = g(3, 3, -1, 0);
+            s0 = mid(0, e0, e1, e2, e3);
+            s1 = mid(1, e0, e1, e2, e3);
+        }
+        out[0][0] = sub(out[0][0], s0);
+        out[0][1] = sub(out[0][1], s1);
     }
     if (down) {    // row 0 of the tile below: +dT[0][v]
-        const V e0 = g(0, 0, 1, 0), e1 = g(0, 1, 1, 0), e2 = g(0, 2, 1, 0), e3 = g(0, 3, 1, 0);
-        out[1][0] = add(out[1][0], mid(0, e0, e1, e2, e3));
-        out[1][1] = add(out[1][1], mid(1, e0, e1, e2, e3));
+        V s0, s1;
+        if (inside(1, 0)) {
+            s0 = ex[IG_TO_ABOVE][threadIdx.x + nb(1, 0)];
+            s1 = ex[IG_TO_ABOVE + 1][threadIdx.x + nb(1, 0)];
+        } else {
+            const V e0 = g(0, 0, 1, 0), e1 = g(0, 1, 1, 0), e2 = g(0, 2, 1, 0), e3 = g(0, 3, 1, 0);
+            s0 = mid(0, e0, e1, e2, e3);
+            s1 = mid(1, e0, e1, e2, e3);
+        }
+        out[1][0] = add(out[1][0], s0);
+        out[1][1] = add(out[1][1], s1);
     }
     if (left) {    // column 3 of the tile to the left: -dT[u][3]
-        const V e0 = g(0, 3, 0, -1), e1 = g(1, 3, 0, -1), e2 = g(2, 3, 0, -1), e3 = g(3, 3, 0, -1);
-        out[0][0] = sub(out[0][0], mid(0, e0, e1, e2, e3));
-        out[1][0] = sub(out[1][0], mid(1, e0, e1, e2, e3));
+        V s0, s1;
+        if (inside(0, -1)) {
+            s0 = ex[IG_TO_RIGHT][threadIdx.x + nb(0, -1)];
+            s1 = ex[IG_TO_RIGHT + 1][threadIdx.x + nb(0, -1)];
+        } else {
+            const V e0 = g(0, 3, 0, -1), e1 = g(1, 3, 0, -1), e2 = g(2, 3, 0, -1), e3 = g(3, 3, 0, -1);
+            s0 = mid(0, e0, e1, e2, e3);
+            s1 = mid(1, e0, e1, e2, e3);
+        }
+        out[0][0] = sub(out[0][0], s0);
+        out[1][0] = sub(out[1][0], s1);
     }
     if (right) {   // column 0 of the tile to the right: +dT[u][0]
-        const V e0 = g(0, 0, 0, 1), e1 = g(1, 0, 0, 1), e2 = g(2, 0, 0, 1), e3 = g(3, 0, 0, 1);
-        out[0][1] = add(out[0][1], mid(0, e0, e1, e2, e3));
-        out[1][1] = add(out[1][1], mid(1, e0, e1, e2, e3));
+        V s0, s1;
+        if (inside(0, 1)) {
+            s0 = ex[IG_TO_LEFT][threadIdx.x + nb(0, 1)];
+            s1 = ex[IG_TO_LEFT + 1][threadIdx.x + nb(0, 1)];
+        } else {
+            const V e0 = g(0, 0, 0, 1), e1 = g(1, 0, 0, 1), e2 = g(2, 0, 0, 1), e3 = g(3, 0, 0, 1);
+            s0 = mid(0, e0, e1, e2, e3);
+            s1 = mid(1, e0, e1, e2, e3);
+        }
+        out[0][1] = add(out[0][1], s0);
+        out[1][1] = add(out[1][1], s1);
     }
     // corners: (-1)(-1) dT[3][3], (-1)(+1) dT[3][0], (+1)(-1) dT[0][3], (+1)(+1) dT[0][0]
-    if (up && left) out[0][0] = add(out[0][0], g(3, 3, -1, -1));
-    if (up && right) out[0][1] = sub(out[0][1], g(3, 0, -1, 1));
-    if (down && left) out[1][0] = sub(out[1][0], g(0, 3, 1, -1));
-    if (down && right) out[1][1] = add(out[1][1], g(0, 0, 1, 1));
+    if (up && left) out[0][0] = add(out[0][0], inside(-1, -1) ? ex[IG_C33][threadIdx.x + nb(-1, -1)] : g(3, 3, -1, -1));
+    if (up && right) out[0][1] = sub(out[0][1], inside(-1, 1) ? ex[IG_C30][threadIdx.x + nb(-1, 1)] : g(3, 0, -1, 1));
+    if (down && left) out[1][0] = sub(out[1][0], inside(1, -1) ? ex[IG_C03][threadIdx.x + nb(1, -1)] : g(0, 3, 1, -1));
+    if (down && right) out[1][1] = add(out[1][1], inside(1, 1) ? ex[IG_C00][threadIdx.x + nb(1, 1)] : g(0, 0, 1, 1));
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
@@ -280,11 +356,32 @@ extern "C" int swc_winograd2x2_imtrans_grad(const float *TransIm_grad, const flo
     const bool vec = (C % 4 == 0) && aligned16(TransIm_grad) && aligned16(Input_grad) &&
                      (relu_mask_source == nullptr || aligned16(relu_mask_source));
     // one lane per (tile, channel vector): each writes the four pixels its tile is centred on
-    const unsigned items = static_cast<unsigned>(static_cast<size_t>(B) * nH * nW * (vec ? C / 4 : C));
-    const dim3 grid((items + 255) / 256), block(256);
+    const unsigned CV = static_cast<unsigned>(vec ? C / 4 : C);
+    const unsigned cgroups = (CV + IG_LANES - 1) / IG_LANES;
+    // Block shape: the one that reads the fewest planes.  A block of rh x rw tiles reads 16 planes per
+    // tile and 4 per tile of its rim; lanes beyond the image's edge idle (weighted a quarter of a read).
+    int rw_shift = 0;
+    unsigned blocks_x = 0, blocks_y = 0;
+    double best = 0;
+    for (int sh = 0; (1 << sh) <= IG_TILES; ++sh) {
+        const int rw = 1 << sh, rh = IG_TILES >> sh;
+        const unsigned bx = (nW + rw - 1) / rw, by = (nH + rh - 1) / rh;
+        const double blocks = static_cast<double>(bx) * by;
+        const double cost = blocks * (2 * (rw < nW ? rw : nW) * (by > 1) + 2 * (rh < nH ? rh : nH) * (bx > 1)) * 4 +
+                            (blocks * IG_TILES - static_cast<double>(nH) * nW) * 4;
+        if (blocks_x == 0 || cost <= best) {  // ties go to the wider block
+            best = cost;
+            rw_shift = sh;
+            blocks_x = bx;
+            blocks_y = by;
+        }
+    }
+    const size_t wgs = static_cast<size_t>(cgroups) * blocks_x * blocks_y * B;
+    if (wgs >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
+    const dim3 grid(static_cast<unsigned>(wgs)), block(IG_THREADS);
 #define SWC_LAUNCH(VEC, MASK)                                                                                   \
     imtrans_grad_tile_kernel<VEC, MASK><<<grid, block, 0, s>>>(TransIm_grad, relu_mask_source, Input_grad, H, W, C, \
-                                                               nH, nW, items, plane)
+                                                               nH, nW, cgroups, blocks_x, blocks_y, rw_shift, plane)
     if (vec) {
         if (relu_mask_source) SWC_LAUNCH(4, true); else SWC_LAUNCH(4, false);
     } else {

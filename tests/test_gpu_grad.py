@@ -28,6 +28,8 @@ def gpu(a, dev):
 
 @pytest.mark.parametrize("shape", [
     (2, 6, 6, 8), (2, 7, 5, 4), (1, 8, 4, 3), (1, 1, 1, 1), (4, 28, 28, 128), (2, 14, 14, 36),
+    # several workgroup blocks of tiles along one axis, ragged at the far edge:
+    (1, 9, 139, 8), (2, 141, 5, 4), (1, 37, 43, 12),
 ])
 @pytest.mark.parametrize("masked", [False, True])
 def test_imtrans_grad(oracle, dev, shape, masked):
