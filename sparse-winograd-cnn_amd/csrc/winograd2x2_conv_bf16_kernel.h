@@ -38,22 +38,23 @@ struct HbCfg {
     static_assert((NSTAGE - 2) * COPIES < 64, "vmcnt range");
 };
 
-// Requires C % BK == 0 and 16-byte aligned TI16 / Wt16.  M < 2^31.
+// Requires C % BK == 0 and 16-byte aligned TI16 / Wt16.  M < 2^31.  grid.x = ceil(M / rows_per_wg) * tiles_n.
 // ABL: timing ablations for development (bit 0: no barrier, 1: no copy wait, 2: no copies, 3: no LDS
 // reads, 4: no MFMA); results are wrong with any bit set.  Always 0 in the library.
 template <typename Cfg, int ABL = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_bf16_stored_kernel(
     const unsigned short *__restrict__ TI16, const unsigned short *__restrict__ Wt16, float *__restrict__ Out, size_t M,
-    int C, int K, int nH, int nW, unsigned tiles_n, ConvEpilogue ep)
+    int C, int K, int nH, int nW, unsigned tiles_n, unsigned rows_per_wg, ConvEpilogue ep)
 {
     constexpr int BK = Cfg::BK, NSTAGE = Cfg::NSTAGE, CH = Cfg::CH, RPC = Cfg::ROWS_PER_COPY, PW = Cfg::PER_WAVE;
     constexpr int ROW_BYTES = BK * 2;
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem_b[];
 
     const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
-    const size_t m0 = static_cast<size_t>(lid / tiles_n) * HB_BM;
+    // A workgroup takes rows_per_wg <= HB_BM rows (the launcher levels the load over the CUs with it).
+    const size_t m0 = static_cast<size_t>(lid / tiles_n) * rows_per_wg;
     const int n0 = static_cast<int>(lid % tiles_n) * HB_BN;
-    const unsigned rows_valid = static_cast<unsigned>(M - m0 < HB_BM ? M - m0 : HB_BM);
+    const unsigned rows_valid = static_cast<unsigned>(M - m0 < rows_per_wg ? M - m0 : rows_per_wg);
     const unsigned cols_valid = static_cast<unsigned>(K - n0 < HB_BN ? K - n0 : HB_BN);
 
     const int tid = threadIdx.x, lane = tid & 63;
