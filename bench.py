@@ -444,7 +444,7 @@ def main():
         dy = torch.randn(B, 2 * nH, 2 * nW, K, device=dev)
         dti, dw = torch.empty_like(ti), torch.empty_like(w)
         tmp = torch.empty(16 * M * K, device=dev)
-        dx = torch.empty(B, 2 * nH, 2 * nW, C, device=dev)
+        dx = torch.empty(B, H, W, C, device=dev)
         ptr = lambda t: t.data_ptr()  # noqa: E731
 
         def f_conv_grad():
@@ -452,22 +452,32 @@ def main():
                                            1, 1, stream) != 0:
                 raise RuntimeError("swc_winograd2x2_conv_grad failed")
 
-        def f_imtrans_grad():
-            if L.swc_winograd2x2_imtrans_grad(ptr(dti), tip, ptr(dx), C, B, 2 * nH, 2 * nW, 1, 1, stream) != 0:
+        def f_imtrans_grad():   # ReLU mask read from the forward result (TI)
+            if L.swc_winograd2x2_imtrans_grad(ptr(dti), tip, ptr(dx), C, B, H, W, 1, 1, stream) != 0:
                 raise RuntimeError("swc_winograd2x2_imtrans_grad failed")
+
+        def f_imtrans_grad_input():   # ReLU mask recomputed from the forward input: what the autograd path calls
+            if L.swc_winograd2x2_imtrans_grad_relu_input(ptr(dti), xp, ptr(dx), C, B, H, W, 1, 1, stream) != 0:
+                raise RuntimeError("swc_winograd2x2_imtrans_grad_relu_input failed")
 
         for _ in range(3):
             f_conv_grad()
             f_imtrans_grad()
+            f_imtrans_grad_input()
         iters = max(args.steps // 4, 10)
         ms_cg = time_loop(f_conv_grad, iters, torch)
         ms_ig = time_loop(f_imtrans_grad, iters, torch)
+        ms_igx = time_loop(f_imtrans_grad_input, iters, torch)
+        dx_bytes = 4.0 * B * H * W * C
         out["backward"] = {
             "ms_conv_grad": round(ms_cg, 5),
             "conv_grad_TFLOPs": round(2 * gemm_flops / (ms_cg * 1e-3) / 1e12, 2),  # two GEMMs of 32*M*C*K each
-            "ms_imtrans_grad": round(ms_ig, 5),
-            # reads dT and the mask source (2 * 64*M*C bytes), writes dX
-            "imtrans_grad_GBps": round((128.0 * M * C + 4.0 * B * 4 * nH * nW * C) / (ms_ig * 1e-3) / 1e9, 1),
+            # reads dT and the forward input (64*M*C + |X| bytes), writes dX
+            "ms_imtrans_grad": round(ms_igx, 5),
+            "imtrans_grad_GBps": round((64.0 * M * C + 2 * dx_bytes) / (ms_igx * 1e-3) / 1e9, 1),
+            # reads dT and the forward result as the mask source (2 * 64*M*C bytes), writes dX
+            "ms_imtrans_grad_mask_from_output": round(ms_ig, 5),
+            "imtrans_grad_mask_from_output_GBps": round((128.0 * M * C + dx_bytes) / (ms_ig * 1e-3) / 1e9, 1),
         }
 
     if not args.no_cpu:

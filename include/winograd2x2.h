@@ -265,6 +265,18 @@ SWC_API int swc_winograd2x2_imtrans_grad(const float *TransIm_grad, const float 
                                          float *Input_grad, int C, int B, int H, int W,
                                          int pad_h, int pad_w, swc_stream_t stream);
 
+/*
+ * The same gradient through the fused ReLU, with the ReLU's mask recomputed from the forward
+ * op's input instead of read from its output: Input [B,H,W,C] is what swc_winograd2x2_imtrans was
+ * given (no scale/shift), and the transform's additions are repeated in the forward order, so the
+ * mask is the forward pass's bit for bit.  Reads a quarter of the bytes the mask costs above and
+ * lets a training caller keep [B,H,W,C] instead of [16,B,nH,nW,C] for this op's backward.
+ * No counterpart in the reference, whose ReLU is a separate op (ResNet-18-var/winograd_imtrans.py:17).
+ */
+SWC_API int swc_winograd2x2_imtrans_grad_relu_input(const float *TransIm_grad, const float *Input,
+                                                    float *Input_grad, int C, int B, int H, int W,
+                                                    int pad_h, int pad_w, swc_stream_t stream);
+
 #ifdef __cplusplus
 } /* extern "C" */
 

@@ -81,6 +81,31 @@ __global__ __launch_bounds__(256) void output_transform_grad_kernel(const float 
 // and the same combination over v for the column, the own tile needs all 16 planes once, each edge
 // neighbour one row or column of 4 planes and each corner one plane: 36 loads for 4 pixels where the
 // per-pixel form issues 64.
+// Plane p of B^T d B from the 16 pixels of a patch, as the forward kernel evaluates it: the four
+// terms of winograd2x2_imTrans_cuda.cu.cc:112-127 added left to right (only additions, so the value
+// and its sign are those of the forward pass bit for bit).  ld(j) yields pixel j = 4r + s.
+template <typename V, typename L>
+__device__ __forceinline__ V plane_of_patch(int p, L ld)
+{
+    constexpr signed char term[16][4] = {{0, 2, 8, 10},  {1, 2, 9, 10},  {2, 1, 9, 10},   {1, 3, 9, 11},
+                                         {4, 6, 8, 10},  {5, 6, 9, 10},  {6, 5, 9, 10},   {5, 7, 9, 11},
+                                         {6, 4, 8, 10},  {9, 6, 5, 10},  {5, 6, 9, 10},   {7, 5, 9, 11},
+                                         {4, 6, 12, 14}, {5, 6, 13, 14}, {6, 5, 13, 14},  {5, 7, 13, 15}};
+    constexpr signed char sign[16][3] = {{-1, -1, 1}, {1, -1, -1}, {-1, 1, -1}, {-1, -1, 1},
+                                         {-1, 1, -1}, {1, 1, 1},   {-1, -1, 1}, {-1, 1, -1},
+                                         {-1, 1, -1}, {-1, -1, 1}, {-1, -1, 1}, {-1, 1, -1},
+                                         {-1, -1, 1}, {1, -1, -1}, {-1, 1, -1}, {-1, -1, 1}};
+    V t = ld(term[p][0]);
+#pragma unroll
+    for (int q = 0; q < 3; ++q) t = sign[p][q] > 0 ? add(t, ld(term[p][q + 1])) : sub(t, ld(term[p][q + 1]));
+    return t;
+}
+
+// How the gradient is masked: not at all, by the sign of the forward result (mask_src = TI), or by
+// the sign of the forward result recomputed from the forward input (mask_src = X [B,H,W,C], a
+// quarter of TI's bytes).
+enum { IG_NO_MASK = 0, IG_MASK_TI = 1, IG_MASK_INPUT = 2 };
+
 // A workgroup takes a block of IG_TILES tiles of one image, rh rows by rw = 1 << rw_shift columns,
 // and IG_LANES channel vectors of each.  Every lane loads its own tile's 16 planes once and leaves in
 // LDS the 12 sums its neighbours need of them (two per edge, one per corner); a neighbour inside the
@@ -95,7 +120,7 @@ constexpr int IG_TILES = IG_THREADS / IG_LANES;
 enum { IG_TO_BELOW = 0, IG_TO_ABOVE = 2, IG_TO_RIGHT = 4, IG_TO_LEFT = 6, IG_C33 = 8, IG_C30 = 9, IG_C03 = 10, IG_C00 = 11, IG_SLOTS = 12 };
 
 // grid.x = cgroups * blocks_x * blocks_y * B
-template <int VEC, bool MASK>
+template <int VEC, int MASK>
 __global__ __launch_bounds__(IG_THREADS) void imtrans_grad_tile_kernel(const float *__restrict__ dT,
                                                                        const float *__restrict__ mask_src,
                                                                        float *__restrict__ dX, int H, int W, int C, int nH,
@@ -118,13 +143,22 @@ __global__ __launch_bounds__(IG_THREADS) void imtrans_grad_tile_kernel(const flo
     const int ty = tl >> rw_shift, tx = tl & (rw - 1);
     const int th = static_cast<int>(byi) * rh + ty, tw = static_cast<int>(bxi) * rw + tx;
     const bool valid = th < nH && tw < nW && cv < CV;
+    // pixel j = 4r + s of the patch of tile (th+dy, tw+dx) of the forward input, zero outside the image
+    auto pixel = [&](int dy, int dx, int j) __attribute__((always_inline)) -> V {
+        const int y = 2 * (th + dy) - 1 + j / 4, x = 2 * (tw + dx) - 1 + j % 4;
+        V d = {};
+        if (y >= 0 && y < H && x >= 0 && x < W)
+            d = *reinterpret_cast<const V *>(mask_src + ((static_cast<size_t>(b) * H + y) * W + x) * C + static_cast<size_t>(cv) * VEC);
+        return d;
+    };
     // masked gradient of plane 4u+v at tile (th+dy, tw+dx)
     auto g = [&](int u, int v, int dy, int dx) __attribute__((always_inline)) -> V {
         const size_t off = static_cast<size_t>(4 * u + v) * plane +
                            ((static_cast<size_t>(b) * nH + (th + dy)) * nW + (tw + dx)) * C + static_cast<size_t>(cv) * VEC;
         V x = *reinterpret_cast<const V *>(dT + off);
-        if (MASK) {
-            const V t = *reinterpret_cast<const V *>(mask_src + off);
+        if (MASK != IG_NO_MASK) {
+            const V t = MASK == IG_MASK_TI ? *reinterpret_cast<const V *>(mask_src + off)
+                                           : plane_of_patch<V>(4 * u + v, [&](int j) __attribute__((always_inline)) { return pixel(dy, dx, j); });
             float *xp = reinterpret_cast<float *>(&x);
             const float *tp = reinterpret_cast<const float *>(&t);
 #pragma unroll
@@ -139,10 +173,37 @@ __global__ __launch_bounds__(IG_THREADS) void imtrans_grad_tile_kernel(const flo
     V out[2][2];
     if (valid) {   // own tile: rows 1+a, then columns 1+b; and what the neighbours need of it
         V t[4][4];
+        if (MASK == IG_MASK_INPUT) {
+            // the own tile's patch is loaded once; bit p of keep[q] says whether plane p passed the ReLU
+            unsigned keep[VEC] = {};
+            {
+                V d[16];
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+                for (int j = 0; j < 16; ++j) d[j] = pixel(0, 0, j);
 #pragma unroll
-            for (int v = 0; v < 4; ++v) t[u][v] = g(u, v, 0, 0);
+                for (int p = 0; p < 16; ++p) {
+                    const V tp = plane_of_patch<V>(p, [&](int j) __attribute__((always_inline)) { return d[j]; });
+                    const float *tq = reinterpret_cast<const float *>(&tp);
+#pragma unroll
+                    for (int q = 0; q < VEC; ++q) keep[q] |= (tq[q] > 0.f ? 1u : 0u) << p;
+                }
+            }
+#pragma unroll
+            for (int p = 0; p < 16; ++p) {
+                const size_t off = static_cast<size_t>(p) * plane +
+                                   ((static_cast<size_t>(b) * nH + th) * nW + tw) * C + static_cast<size_t>(cv) * VEC;
+                V x = *reinterpret_cast<const V *>(dT + off);
+                float *xp = reinterpret_cast<float *>(&x);
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) xp[q] = (keep[q] >> p) & 1u ? xp[q] : 0.f;
+                t[p / 4][p % 4] = x;
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) t[u][v] = g(u, v, 0, 0);
+        }
         V row[2][4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
@@ -341,10 +402,13 @@ extern "C" int swc_winograd2x2_conv_grad(const float *TInput, const float *Weigh
     return rs == rocblas_status_success ? SWC_OK : SWC_ERR_HIP;
 }
 
-extern "C" int swc_winograd2x2_imtrans_grad(const float *TransIm_grad, const float *relu_mask_source, float *Input_grad,
-                                            int C, int B, int H, int W, int pad_h, int pad_w, swc_stream_t stream)
+namespace swc {
+namespace {
+// mask_mode: IG_NO_MASK (mask_source unused), IG_MASK_TI (mask_source = the forward result [16,B,nH,nW,C]) or
+// IG_MASK_INPUT (mask_source = the forward input [B,H,W,C]).
+int imtrans_grad_entry(const float *TransIm_grad, const float *relu_mask_source, int mask_mode, float *Input_grad, int C,
+                       int B, int H, int W, int pad_h, int pad_w, swc_stream_t stream)
 {
-    using namespace swc;
     if (TransIm_grad == nullptr || Input_grad == nullptr) return SWC_ERR_NULL_POINTER;
     if (C <= 0 || B <= 0 || H <= 0 || W <= 0) return SWC_ERR_BAD_DIMS;
     if (pad_h != 1 || pad_w != 1) return SWC_ERR_BAD_PAD;
@@ -383,13 +447,35 @@ extern "C" int swc_winograd2x2_imtrans_grad(const float *TransIm_grad, const flo
     imtrans_grad_tile_kernel<VEC, MASK><<<grid, block, 0, s>>>(TransIm_grad, relu_mask_source, Input_grad, H, W, C, \
                                                                nH, nW, cgroups, blocks_x, blocks_y, rw_shift, plane)
     if (vec) {
-        if (relu_mask_source) SWC_LAUNCH(4, true); else SWC_LAUNCH(4, false);
+        if (mask_mode == IG_MASK_TI) SWC_LAUNCH(4, IG_MASK_TI);
+        else if (mask_mode == IG_MASK_INPUT) SWC_LAUNCH(4, IG_MASK_INPUT);
+        else SWC_LAUNCH(4, IG_NO_MASK);
     } else {
-        if (relu_mask_source) SWC_LAUNCH(1, true); else SWC_LAUNCH(1, false);
+        if (mask_mode == IG_MASK_TI) SWC_LAUNCH(1, IG_MASK_TI);
+        else if (mask_mode == IG_MASK_INPUT) SWC_LAUNCH(1, IG_MASK_INPUT);
+        else SWC_LAUNCH(1, IG_NO_MASK);
     }
 #undef SWC_LAUNCH
     return check_launch();
 }
+}  // namespace
+}  // namespace swc
+
+extern "C" int swc_winograd2x2_imtrans_grad(const float *TransIm_grad, const float *relu_mask_source, float *Input_grad,
+                                            int C, int B, int H, int W, int pad_h, int pad_w, swc_stream_t stream)
+{
+    return swc::imtrans_grad_entry(TransIm_grad, relu_mask_source, relu_mask_source ? swc::IG_MASK_TI : swc::IG_NO_MASK,
+                                   Input_grad, C, B, H, W, pad_h, pad_w, stream);
+}
+
+extern "C" int swc_winograd2x2_imtrans_grad_relu_input(const float *TransIm_grad, const float *Input, float *Input_grad,
+                                                       int C, int B, int H, int W, int pad_h, int pad_w,
+                                                       swc_stream_t stream)
+{
+    if (Input == nullptr) return SWC_ERR_NULL_POINTER;
+    return swc::imtrans_grad_entry(TransIm_grad, Input, swc::IG_MASK_INPUT, Input_grad, C, B, H, W, pad_h, pad_w, stream);
+}
+
 
 void Winograd2x2ConvGradComputeLauncher(const float *TInput, const float *Weight, const float *Output_grad,
                                         float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,

@@ -27,7 +27,8 @@ C_SYMBOLS = (
     "swc_winograd2x2_relu_conv_bf16",
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
-    "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad", "swc_winograd2x2_relu_conv",
+    "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad", "swc_winograd2x2_imtrans_grad_relu_input",
+    "swc_winograd2x2_relu_conv",
 )
 # The two C++-linkage launchers with the reference's exact signatures (Itanium mangling).
 CXX_SYMBOLS = (
@@ -104,6 +105,8 @@ def lib():
         L.swc_winograd2x2_conv_grad.argtypes = [fp] * 7 + [i32] * 7 + [vp]
         L.swc_winograd2x2_imtrans_grad.restype = i32
         L.swc_winograd2x2_imtrans_grad.argtypes = [fp] * 3 + [i32] * 6 + [vp]
+        L.swc_winograd2x2_imtrans_grad_relu_input.restype = i32
+        L.swc_winograd2x2_imtrans_grad_relu_input.argtypes = [fp] * 3 + [i32] * 6 + [vp]
         _lib = L
     return _lib
 

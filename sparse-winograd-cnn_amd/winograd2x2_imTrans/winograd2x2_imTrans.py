@@ -59,17 +59,29 @@ def _forward(I, relu, out, scale=None, shift=None, out_dtype=torch.float32):
     return out
 
 
-def winograd2x2_imTrans_grad(grad, H=None, W=None, relu_output=None):
+def winograd2x2_imTrans_grad(grad, H=None, W=None, relu_output=None, relu_input=None):
     """grad: [16,B,nH,nW,C] -> gradient w.r.t. the op's input, [B,H,W,C].
 
     As in the reference (winograd2x2_imTrans_grad_op.cc:44-45) H and W default to 2*nH, 2*nW.
-    ``relu_output``: the forward result computed with ``relu=True``; the gradient is then taken
-    through the fused ReLU.  ``grad`` is left untouched (the reference overwrites it).
+    The gradient is taken through the fused ReLU when the forward pass's result (``relu_output``,
+    computed with ``relu=True``) or its input (``relu_input`` [B,H,W,C]; the mask is recomputed from
+    it, which reads a quarter of the bytes) is given.  ``grad`` is left untouched (the reference
+    overwrites it).
     """
     grad = swc_hip.require_cuda_f32(grad, "grad", 5)
     if grad.shape[0] != 16:
         raise ValueError("grad must have shape [16,B,nH,nW,C]")
     _, B, nH, nW, C = grad.shape
+    if relu_input is not None:
+        if relu_output is not None:
+            raise ValueError("give relu_output or relu_input, not both")
+        relu_input = swc_hip.require_cuda_f32(relu_input, "relu_input", 4)
+        if relu_input.shape[0] != B or relu_input.shape[3] != C:
+            raise ValueError("relu_input must be the forward input [B,H,W,C]")
+        H = relu_input.shape[1] if H is None else int(H)
+        W = relu_input.shape[2] if W is None else int(W)
+        if (H, W) != tuple(relu_input.shape[1:3]):
+            raise ValueError("relu_input is %d x %d, not %d x %d" % (relu_input.shape[1], relu_input.shape[2], H, W))
     H = 2 * nH if H is None else int(H)
     W = 2 * nW if W is None else int(W)
     if (H + 1) // 2 != nH or (W + 1) // 2 != nW:
@@ -82,8 +94,13 @@ def winograd2x2_imTrans_grad(grad, H=None, W=None, relu_output=None):
         mask_ptr = relu_output.data_ptr()
     out = torch.empty((B, H, W, C), dtype=torch.float32, device=grad.device)
     with torch.cuda.device(grad.device):
-        st = swc_hip.lib().swc_winograd2x2_imtrans_grad(grad.data_ptr(), mask_ptr, out.data_ptr(), C, B, H, W, 1, 1,
-                                                        torch.cuda.current_stream().cuda_stream)
+        stream = torch.cuda.current_stream().cuda_stream
+        if relu_input is not None:
+            st = swc_hip.lib().swc_winograd2x2_imtrans_grad_relu_input(grad.data_ptr(), relu_input.data_ptr(),
+                                                                       out.data_ptr(), C, B, H, W, 1, 1, stream)
+        else:
+            st = swc_hip.lib().swc_winograd2x2_imtrans_grad(grad.data_ptr(), mask_ptr, out.data_ptr(), C, B, H, W, 1, 1,
+                                                            stream)
     swc_hip.check(st, "winograd2x2_imTrans_grad")
     return out
 
@@ -97,13 +114,14 @@ class _ImTransFunction(torch.autograd.Function):
         ctx.hw = (I.shape[1], I.shape[2])
         ctx.relu = bool(relu)
         if relu:
-            ctx.save_for_backward(out)
+            # the ReLU's mask is recomputed from the input in the backward pass: [B,H,W,C] kept, not [16,B,nH,nW,C]
+            ctx.save_for_backward(I)
         return out
 
     @staticmethod
     def backward(ctx, grad):
-        relu_output = ctx.saved_tensors[0] if ctx.relu else None
-        return winograd2x2_imTrans_grad(grad.contiguous(), ctx.hw[0], ctx.hw[1], relu_output), None
+        relu_input = ctx.saved_tensors[0] if ctx.relu else None
+        return winograd2x2_imTrans_grad(grad.contiguous(), ctx.hw[0], ctx.hw[1], relu_input=relu_input), None
 
 
 def winograd2x2_imTrans(I, relu=False, out=None, scale=None, shift=None, out_dtype=torch.float32):

@@ -31,22 +31,48 @@ def gpu(a, dev):
     # several workgroup blocks of tiles along one axis, ragged at the far edge:
     (1, 9, 139, 8), (2, 141, 5, 4), (1, 37, 43, 12),
 ])
-@pytest.mark.parametrize("masked", [False, True])
+@pytest.mark.parametrize("masked", [False, True, "input"])
 def test_imtrans_grad(oracle, dev, shape, masked):
+    """masked: through the fused ReLU, with its mask read from the forward result (True) or recomputed
+    from the forward input ("input"; must give the same bits)."""
     from winograd2x2_imTrans.winograd2x2_imTrans import winograd2x2_imTrans_grad
     B, H, W, C = shape
     rng = np.random.default_rng(31)
     x = rng.standard_normal(shape).astype(np.float32)
+    if masked == "input":
+        # values whose sums cancel exactly, so that entries of the transform sit at 0 (masked) and not near it
+        x = rng.integers(-2, 3, size=shape).astype(np.float32)
     ti = oracle.imtrans(x, relu=True)
+    kw = {}
+    if masked is True:
+        kw["relu_output"] = gpu(ti, dev)
+    elif masked == "input":
+        kw["relu_input"] = gpu(x, dev)
     g = rng.standard_normal(ti.shape).astype(np.float32)
     want = oracle.imtrans_grad(g, H, W, mask_src=ti if masked else None)
-    got = winograd2x2_imTrans_grad(gpu(g, dev), H, W, gpu(ti, dev) if masked else None).cpu().numpy()
+    got = winograd2x2_imTrans_grad(gpu(g, dev), H, W, **kw).cpu().numpy()
     assert got.shape == (B, H, W, C)
     assert rel_max(got, want) <= 1e-6
     gi = rng.integers(-4, 5, size=ti.shape).astype(np.float32)
     wanti = oracle.imtrans_grad(gi, H, W, mask_src=ti if masked else None)
-    goti = winograd2x2_imTrans_grad(gpu(gi, dev), H, W, gpu(ti, dev) if masked else None).cpu().numpy()
+    goti = winograd2x2_imTrans_grad(gpu(gi, dev), H, W, **kw).cpu().numpy()
     assert np.array_equal(goti, wanti)
+
+
+def test_imtrans_grad_mask_from_input_matches_mask_from_output(dev):
+    """On real-valued inputs the recomputed mask is the forward pass's own, bit for bit."""
+    from winograd2x2_imTrans.winograd2x2_imTrans import winograd2x2_imTrans, winograd2x2_imTrans_grad
+    torch.manual_seed(5)
+    x = torch.randn(3, 13, 27, 20, device=dev)
+    ti = winograd2x2_imTrans(x, relu=True)
+    g = torch.randn_like(ti)
+    a = winograd2x2_imTrans_grad(g, 13, 27, relu_output=ti)
+    b = winograd2x2_imTrans_grad(g, relu_input=x)
+    assert torch.equal(a, b)
+    with pytest.raises(ValueError):
+        winograd2x2_imTrans_grad(g, relu_output=ti, relu_input=x)
+    with pytest.raises(ValueError):
+        winograd2x2_imTrans_grad(g, relu_input=x[:, :12])
 
 
 @pytest.mark.parametrize("shape", [
