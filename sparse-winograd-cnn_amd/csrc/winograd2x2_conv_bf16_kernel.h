@@ -40,7 +40,7 @@ struct HbCfg {
 
 // Requires C % BK == 0 and 16-byte aligned TI16 / Wt16.  M < 2^31.  grid.x = ceil(M / rows_per_wg) * tiles_n.
 // ABL: timing ablations for development (bit 0: no barrier, 1: no copy wait, 2: no copies, 3: no LDS
-// reads, 4: no MFMA); results are wrong with any bit set.  Always 0 in the library.
+// reads, 4: no MFMA, 6: no output stores); results are wrong with any bit set.  Always 0 in the library.
 template <typename Cfg, int ABL = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_bf16_stored_kernel(
     const unsigned short *__restrict__ TI16, const unsigned short *__restrict__ Wt16, float *__restrict__ Out, size_t M,
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
     });
     wait_vmcnt<0>();  // the surplus copies must land before the workgroup's LDS is handed on
 
-    store_output<HbStoreCfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
+    if (!(ABL & 64) || nH < 0) store_output<HbStoreCfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
 }
 
 // W [16,C,K] fp32 -> Wt16 [16,K,C] bf16 (round to nearest even).  One lane per output element.
