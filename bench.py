@@ -133,19 +133,57 @@ def bench_resnet(args, torch, dev):
     sizes = {"2": 56, "3": 28, "4": 14, "5": 14}
     flops = sum(18.0 * N * sizes[n[len("Winograd_W")]] ** 2 * c.in_channel * c.out_channel
                 for n, c in zip(resnet18_var.winograd_layer_names(), model.winograd_convs()))
-    for _ in range(max(args.warmup // 4, 2)):
-        logits = model(image)
-    torch.cuda.synchronize()
-    steps = max(args.steps // 10, 5)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        logits = model(image)
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / steps
+    with torch.no_grad():
+        for _ in range(max(args.warmup // 4, 2)):
+            logits = model(image)
+        torch.cuda.synchronize()
+        steps = max(args.steps // 10, 5)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            logits = model(image)
+        torch.cuda.synchronize()
+        ms_eager = (time.perf_counter() - t0) * 1e3 / steps
+        # The same forward replayed from one captured HIP graph: about a hundred launches per forward
+        # (ops of this library and stock PyTorch ones) stop costing host time.  The replay is only
+        # reported if three replays, with eager work between them, each reproduce the eager logits.
+        ms_graph = None
+        if args.graph:
+            try:
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    model(image)
+                torch.cuda.current_stream().wait_stream(side)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    logits_g = model(image)
+                ok = True
+                for _ in range(3):
+                    eager = model(image)
+                    torch.cuda.synchronize()
+                    graph.replay()
+                    torch.cuda.synchronize()
+                    ok = ok and bool(torch.equal(logits_g, eager))
+                if ok:
+                    t0 = time.perf_counter()
+                    for _ in range(steps):
+                        graph.replay()
+                    torch.cuda.synchronize()
+                    ms_graph = (time.perf_counter() - t0) * 1e3 / steps
+                else:
+                    print("bench.py: graph replays of the cfg5 forward differ from the eager result; not reported",
+                          file=sys.stderr)
+            except RuntimeError as e:  # a stock op that cannot be captured
+                print("bench.py: cfg5 forward not captured: %s" % e, file=sys.stderr)
+                torch.cuda.synchronize()
+    ms = ms_eager if ms_graph is None or ms_eager <= ms_graph else ms_graph
     print(json.dumps({
         "metric": "ResNet-18-var Winograd-ReLU forward (config 5), effective conv GFLOP/s of its 16 3x3 layers",
         "value": round(flops / (ms * 1e-3) / 1e9, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": steps,
         "warmup": max(args.warmup // 4, 2), "ms_per_step": round(ms, 3), "images_per_s": round(N / (ms * 1e-3), 1),
+        "launch": "eager" if ms == ms_eager else "graph replay",
+        "ms_per_step_eager": round(ms_eager, 3), "ms_per_step_graph": None if ms_graph is None else round(ms_graph, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"fp32": "f32", "bf16": "bf16 operands, f32 accumulate",
                   "bf16_stored": "bf16 operands (stored as bf16), f32 accumulate"}[args.precision], "data": "synthetic",

@@ -49,6 +49,15 @@ def _same_pad(x, k, stride):
     return pads
 
 
+def _max_pool_same(x):
+    """3x3 stride-2 max-pool with TensorFlow SAME padding.  Where the padding falls entirely behind the
+    data (even sizes) ``ceil_mode`` gives the same windows without a padded copy of the tensor."""
+    pads = _same_pad(x, 3, 2)
+    if pads[0] == 0 and pads[2] == 0:
+        return F.max_pool2d(x, 3, 2, ceil_mode=True)
+    return F.max_pool2d(F.pad(x, pads, value=float("-inf")), 3, 2)
+
+
 def _bn_affine(bn):
     """Inference-mode BatchNorm2d as y = x*scale + shift; cached until a parameter or statistic changes."""
     tensors = (bn.weight, bn.bias, bn.running_mean, bn.running_var)
@@ -58,6 +67,18 @@ def _bn_affine(bn):
         scale = (bn.weight * torch.rsqrt(bn.running_var + bn.eps)).detach()
         cached = (key, scale.contiguous(), (bn.bias - bn.running_mean * scale).detach().contiguous())
         bn._swc_affine = cached
+    return cached[1], cached[2]
+
+
+def _conv_bn_folded(conv, bn):
+    """A bias-free conv followed by an inference-mode BatchNorm as one conv: weights scaled per output
+    channel, the shift as bias.  Cached until the weights or the BatchNorm change."""
+    scale, shift = _bn_affine(bn)
+    key = (conv.weight._version, conv.weight.data_ptr(), bn._swc_affine[0])
+    cached = getattr(conv, "_swc_folded", None)
+    if cached is None or cached[0] != key:
+        cached = (key, (conv.weight * scale.view(-1, 1, 1, 1)).detach(), shift)
+        conv._swc_folded = cached
     return cached[1], cached[2]
 
 
@@ -105,12 +126,16 @@ class WinogradUnit(torch.nn.Module):
     def forward(self, x):
         if self.shortcut:
             s = torch.relu(self.bn_pre(x)) if self.bn_pre is not None else torch.relu(x)
-            sc = self.bn1(self.conv1(s))
+            if self.fold_bn:
+                w1, b1 = _conv_bn_folded(self.conv1, self.bn1)
+                sc = F.conv2d(s, w1, b1)
+            else:
+                sc = self.bn1(self.conv1(s))
         else:
             sc = torch.relu(x)
         x = self.branch(x, sc)
         if self.pool:
-            x = F.max_pool2d(F.pad(x, _same_pad(x, 3, 2), value=float("-inf")), 3, 2)
+            x = _max_pool_same(x)
         return x
 
 
@@ -136,7 +161,7 @@ class ResNet18Var(torch.nn.Module):
         """image: [B,H,W,3] float32 NHWC (already normalised) -> logits [B,num_classes]."""
         x = image.permute(0, 3, 1, 2)  # NCHW view over NHWC memory = channels_last
         x = self.conv1(F.pad(x, _same_pad(x, 7, 2)))
-        x = F.max_pool2d(F.pad(x, _same_pad(x, 3, 2), value=float("-inf")), 3, 2)
+        x = _max_pool_same(x)
         x = x.contiguous(memory_format=torch.channels_last)
         for unit in self.units:
             x = unit(x)
