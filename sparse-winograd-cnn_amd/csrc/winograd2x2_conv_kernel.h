@@ -118,43 +118,62 @@ __device__ __forceinline__ void store_output(const AccT<Cfg> (&Y)[4][Cfg::TM][Cf
     const size_t oW = 2 * static_cast<size_t>(nW);
     const size_t row_stride = oW * K;
     const unsigned m032 = static_cast<unsigned>(m0);
+    // fn(tm, r, tn, element offset of the tile's top-left pixel in this lane's column) for every valid value
+    auto for_each_value = [&](auto fn) __attribute__((always_inline)) {
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
+        for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
-        for (int r = 0; r < Cfg::REGS; ++r) {
-            const unsigned row = wm0 + tm * MF + (MF == 32 ? 8 * (r / 4) + 4 * lg + (r % 4) : 4 * lg + r);
-            if (row >= rows_valid) continue;
-            const unsigned gm = m032 + row;
-            const unsigned bt = gm / static_cast<unsigned>(nW);  // b*nH + th
-            const unsigned tw = gm - bt * static_cast<unsigned>(nW);
-            const size_t pix = (static_cast<size_t>(bt) * 2 * oW + 2 * tw) * K;
-            float *o = Out + pix;
+            for (int r = 0; r < Cfg::REGS; ++r) {
+                const unsigned row = wm0 + tm * MF + (MF == 32 ? 8 * (r / 4) + 4 * lg + (r % 4) : 4 * lg + r);
+                if (row >= rows_valid) continue;
+                const unsigned gm = m032 + row;
+                const unsigned bt = gm / static_cast<unsigned>(nW);  // b*nH + th
+                const unsigned tw = gm - bt * static_cast<unsigned>(nW);
+                const size_t pix = (static_cast<size_t>(bt) * 2 * oW + 2 * tw) * K;
 #pragma unroll
-            for (int tn = 0; tn < TN; ++tn) {
-                const int col = n0 + wn0 + tn * MF + li;
-                if (col >= K) continue;
-                float y0 = Y[0][tm][tn][r], y1 = Y[1][tm][tn][r], y2 = Y[2][tm][tn][r], y3 = Y[3][tm][tn][r];
-                if (affine) {
-                    const float sc = ep.scale[col], sh = ep.shift[col];
-                    y0 = __builtin_fmaf(y0, sc, sh);
-                    y1 = __builtin_fmaf(y1, sc, sh);
-                    y2 = __builtin_fmaf(y2, sc, sh);
-                    y3 = __builtin_fmaf(y3, sc, sh);
+                for (int tn = 0; tn < TN; ++tn) {
+                    const int col = n0 + wn0 + tn * MF + li;
+                    if (col >= K) continue;
+                    fn(tm, r, tn, pix + col);
                 }
-                if (residual) {
-                    const float *q = ep.residual + pix;
-                    y0 += q[col];
-                    y1 += q[K + col];
-                    y2 += q[row_stride + col];
-                    y3 += q[row_stride + K + col];
-                }
-                o[col] = y0;
-                o[K + col] = y1;
-                o[row_stride + col] = y2;
-                o[row_stride + K + col] = y3;
             }
         }
+    };
+    // The residual is read in one sweep before the first store: loads and stores complete in issue
+    // order, so a load issued behind a store also waits for that store, and interleaving them would
+    // cost one memory round trip per group of values instead of one per tile.
+    float q[4][TM][Cfg::REGS][TN];
+    if (residual) {
+        for_each_value([&](int tm, int r, int tn, size_t at) __attribute__((always_inline)) {
+            const float *src = ep.residual + at;
+            q[0][tm][r][tn] = src[0];
+            q[1][tm][r][tn] = src[K];
+            q[2][tm][r][tn] = src[row_stride];
+            q[3][tm][r][tn] = src[row_stride + K];
+        });
     }
+    for_each_value([&](int tm, int r, int tn, size_t at) __attribute__((always_inline)) {
+        float y0 = Y[0][tm][tn][r], y1 = Y[1][tm][tn][r], y2 = Y[2][tm][tn][r], y3 = Y[3][tm][tn][r];
+        if (affine) {
+            const int col = n0 + wn0 + tn * MF + li;
+            const float sc = ep.scale[col], sh = ep.shift[col];
+            y0 = __builtin_fmaf(y0, sc, sh);
+            y1 = __builtin_fmaf(y1, sc, sh);
+            y2 = __builtin_fmaf(y2, sc, sh);
+            y3 = __builtin_fmaf(y3, sc, sh);
+        }
+        if (residual) {
+            y0 += q[0][tm][r][tn];
+            y1 += q[1][tm][r][tn];
+            y2 += q[2][tm][r][tn];
+            y3 += q[3][tm][r][tn];
+        }
+        float *o = Out + at;
+        o[0] = y0;
+        o[K] = y1;
+        o[row_stride] = y2;
+        o[row_stride + K] = y3;
+    });
 }
 
 // FAST: C and K are multiples of 4, TI and Wt 16-byte aligned, and a tile's rows fit 32-bit
