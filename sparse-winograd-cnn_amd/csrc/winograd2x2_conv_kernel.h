@@ -139,20 +139,7 @@ __device__ __forceinline__ void store_output(const AccT<Cfg> (&Y)[4][Cfg::TM][Cf
             }
         }
     };
-    // The residual is read in one sweep before the first store: loads and stores complete in issue
-    // order, so a load issued behind a store also waits for that store, and interleaving them would
-    // cost one memory round trip per group of values instead of one per tile.
-    float q[4][TM][Cfg::REGS][TN];
-    if (residual) {
-        for_each_value([&](int tm, int r, int tn, size_t at) __attribute__((always_inline)) {
-            const float *src = ep.residual + at;
-            q[0][tm][r][tn] = src[0];
-            q[1][tm][r][tn] = src[K];
-            q[2][tm][r][tn] = src[row_stride];
-            q[3][tm][r][tn] = src[row_stride + K];
-        });
-    }
-    for_each_value([&](int tm, int r, int tn, size_t at) __attribute__((always_inline)) {
+    auto finish = [&](int tm, int r, int tn, size_t at, float q0, float q1, float q2, float q3) __attribute__((always_inline)) {
         float y0 = Y[0][tm][tn][r], y1 = Y[1][tm][tn][r], y2 = Y[2][tm][tn][r], y3 = Y[3][tm][tn][r];
         if (affine) {
             const int col = n0 + wn0 + tn * MF + li;
@@ -162,17 +149,44 @@ __device__ __forceinline__ void store_output(const AccT<Cfg> (&Y)[4][Cfg::TM][Cf
             y2 = __builtin_fmaf(y2, sc, sh);
             y3 = __builtin_fmaf(y3, sc, sh);
         }
-        if (residual) {
-            y0 += q[0][tm][r][tn];
-            y1 += q[1][tm][r][tn];
-            y2 += q[2][tm][r][tn];
-            y3 += q[3][tm][r][tn];
-        }
         float *o = Out + at;
-        o[0] = y0;
-        o[K] = y1;
-        o[row_stride] = y2;
-        o[row_stride + K] = y3;
+        o[0] = y0 + q0;
+        o[K] = y1 + q1;
+        o[row_stride] = y2 + q2;
+        o[row_stride + K] = y3 + q3;
+    };
+    if (!residual) {
+        for_each_value([&](int tm, int r, int tn, size_t at) __attribute__((always_inline)) {
+            float y0 = Y[0][tm][tn][r], y1 = Y[1][tm][tn][r], y2 = Y[2][tm][tn][r], y3 = Y[3][tm][tn][r];
+            if (affine) {
+                const int col = n0 + wn0 + tn * MF + li;
+                const float sc = ep.scale[col], sh = ep.shift[col];
+                y0 = __builtin_fmaf(y0, sc, sh);
+                y1 = __builtin_fmaf(y1, sc, sh);
+                y2 = __builtin_fmaf(y2, sc, sh);
+                y3 = __builtin_fmaf(y3, sc, sh);
+            }
+            float *o = Out + at;
+            o[0] = y0;
+            o[K] = y1;
+            o[row_stride] = y2;
+            o[row_stride + K] = y3;
+        });
+        return;
+    }
+    // The residual is read in one sweep before the first store: loads and stores complete in issue
+    // order, so a load issued behind a store also waits for that store, and interleaving them would
+    // cost one memory round trip per group of values instead of one per tile.
+    float q[4][TM][Cfg::REGS][TN];
+    for_each_value([&](int tm, int r, int tn, size_t at) __attribute__((always_inline)) {
+        const float *src = ep.residual + at;
+        q[0][tm][r][tn] = src[0];
+        q[1][tm][r][tn] = src[K];
+        q[2][tm][r][tn] = src[row_stride];
+        q[3][tm][r][tn] = src[row_stride + K];
+    });
+    for_each_value([&](int tm, int r, int tn, size_t at) __attribute__((always_inline)) {
+        finish(tm, r, tn, at, q[0][tm][r][tn], q[1][tm][r][tn], q[2][tm][r][tn], q[3][tm][r][tn]);
     });
 }
 
