@@ -404,7 +404,8 @@ def main():
     gbs_conv = conv_bytes / (ms_conv * 1e-3) / 1e9
     if args.precision == "fp32":
         # fp32 MFMA bounds the contraction (arithmetic intensity 51 flop/B at conv3, ridge 19.7)
-        conv_roofline = {"kernel": "winograd2x2_conv (16 GEMMs + fused A^T m A), fp32 MFMA", "bound": "mfma",
+        conv_roofline = {"kernel": "winograd2x2_conv (16 GEMMs + fused A^T m A), fp32 MFMA, tiling %s"
+                                   % L.swc_winograd2x2_conv_last_kernel().decode(), "bound": "mfma",
                          "achieved": round(tf_conv, 2), "peak": FP32_MFMA_PEAK_TF, "unit": "TFLOP/s",
                          "frac": round(tf_conv / FP32_MFMA_PEAK_TF, 4)}
     else:

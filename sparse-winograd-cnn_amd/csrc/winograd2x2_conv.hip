@@ -132,7 +132,9 @@ int conv_entry(const float *Input, const float *Weight, float *Output, int C, in
         const bool ok32 = async_eligible<Tile32>(Input, Weight, C, K);
         const bool ok_tall = async_eligible<Tall>(Input, Weight, C, K);
         const bool ok_short = async_eligible<Short>(Input, Weight, C, K);
-        const size_t rows_tall = balanced_rows<Tall>(M, tiles_n), rows_short = balanced_rows<Short>(M, tiles_n);
+        // Tall levels its row groups over the CUs; Short does better with full 32-row groups (two whole MFMA
+        // tiles) even where that leaves some CUs with one workgroup more (conv4a: 69 vs 73 us).
+        const size_t rows_tall = balanced_rows<Tall>(M, tiles_n), rows_short = Short::BM;
         const size_t wgs_short = (M + rows_short - 1) / rows_short * tiles_n;
         const double w_short = C < 128 ? 1.15 : wgs_short <= 3 * kCUs ? 0.97 : 1.10;
         const double cost32 = ok32 ? passes((M + 63) / 64 * tiles_n) * 4.0 : 1e30;
