@@ -207,8 +207,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg and the parity gate")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU work for cpu_baseline")
     ap.add_argument("--backward", action="store_true",
-                    help="also time the two gradient ops (conv grad: dP transform + two rocBLAS batched GEMMs; "
-                         "imTrans grad with the ReLU mask) and add a `backward` object to the line")
+                    help="also time the two gradient ops (conv grad: dP transform + the dW and dTI batched GEMMs; "
+                         "imTrans grad through the fused ReLU) and add a `backward` object to the line")
     ap.add_argument("--no-rotate", dest="rotate", action="store_false",
                     help="skip the extra timing over cycled buffer sets (Infinity Cache defeated)")
     ap.add_argument("--no-graph", dest="graph", action="store_false",

@@ -10,10 +10,11 @@
 // where the reference calls cublasSgemmBatched).  dW = TI^T . dP reduces over the tens of thousands
 // of rows of M into a tiny output, a shape the library handles poorly (31 TFLOP/s at ResNet-18
 // conv3); it runs on the split-reduction MFMA kernel of winograd2x2_wgrad_kernel.h, with rocBLAS
-// kept for the shapes that kernel does not take.  ImTrans grad is one gather kernel: every
-// input pixel collects, from the up to 2x2 tiles that cover it, its entry of B dT B^T, recomputed
-// from the (at most 9) transform-domain gradients it depends on; the incoming gradient is not
-// modified (the reference transforms it in place first, :124).
+// kept for the shapes that kernel does not take.  ImTrans grad is one gather kernel: a lane
+// produces the 2x2 input pixels its tile is centred on from the entries of B dT B^T that fall on
+// them -- its own tile's and the up to 8 neighbouring tiles', handed over through LDS inside a
+// workgroup's block of tiles -- optionally through the fused ReLU's mask; the incoming gradient is
+// not modified (the reference transforms it in place first, :124).
 
 #include <cstdio>
 
