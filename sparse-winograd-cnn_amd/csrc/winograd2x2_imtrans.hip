@@ -10,7 +10,6 @@
 // with 48 adds, so HBM bandwidth bounds it.  Channels are the contiguous axis, a lane
 // owns VEC consecutive channels and never needs another lane's data.
 
-#include <cstdlib>
 
 #include "swc_common.h"
 
@@ -70,11 +69,28 @@ struct Vec<4> {
 // 256 MB Infinity Cache, and the pair is 2-3 us slower.  So they are used only when the planes are too
 // large to stay resident anyway (STREAM template flag, chosen by the launcher).
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
+// The planes are written once and read by a later kernel, never by this one, so no store is left as a dirty
+// line in the L2s for the write-back that ends the kernel to drain.
+// fp32 planes: nontemporal stores, streamed past the caches.  With ordinary stores the kernel is 40 % slower
+// once its output no longer fits the Infinity Cache (every line it writes first evicts a dirty one); the fp32
+// convolution that reads the planes next is bound by the matrix pipes and runs equally fast either way.
+// bf16 planes: written through as they are issued (the agent-scope form of a store, sc1) but still allocated
+// in the Infinity Cache, because the bf16 convolution is bound by reading them (its step is 25 % slower when
+// they come from HBM).
 __device__ __forceinline__ void stream_store(float *p, float v) { __builtin_nontemporal_store(v, p); }
 __device__ __forceinline__ void stream_store(float *p, const float4 &v)
 {
     const floatx4_t t = {v.x, v.y, v.z, v.w};
     __builtin_nontemporal_store(t, reinterpret_cast<floatx4_t *>(p));
+}
+__device__ __forceinline__ void through_store(unsigned short *p, unsigned short v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void through_store(unsigned short *p, uint2 v)  // p is 8-byte aligned
+{
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(p), (static_cast<unsigned long long>(v.y) << 32) | v.x,
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 typedef float floatx2_t __attribute__((ext_vector_type(2)));
@@ -84,10 +100,10 @@ __device__ __forceinline__ unsigned pack_bf16(float lo, float hi)
     const bf16x2_t p = __builtin_convertvector(floatx2_t{lo, hi}, bf16x2_t);  // v_cvt_pk_bf16_f32, RNE
     return __builtin_bit_cast(unsigned, p);
 }
-__device__ __forceinline__ void store_bf16(unsigned short *p, float v) { *p = static_cast<unsigned short>(pack_bf16(v, 0.f)); }
+__device__ __forceinline__ void store_bf16(unsigned short *p, float v) { through_store(p, static_cast<unsigned short>(pack_bf16(v, 0.f))); }
 __device__ __forceinline__ void store_bf16(unsigned short *p, const float4 &v)
 {
-    *reinterpret_cast<uint2 *>(p) = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
+    through_store(p, make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w)));
 }
 
 template <int VEC, bool RELU>
@@ -116,7 +132,7 @@ __device__ __forceinline__ void transform_vec(const typename Vec<VEC>::type (&d)
 // AFFINE: every pixel inside the image is first mapped to fma(x, scale[c], shift[c]) (an inference-mode
 // batch normalisation folded into the load); the zero padding stays zero, as it does when the
 // normalisation runs as its own pass before the transform.
-template <int VEC, bool RELU, bool AFFINE, bool STREAM, bool BF16OUT, typename Idx>
+template <int VEC, bool RELU, bool AFFINE, bool BF16OUT, typename Idx>
 __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__restrict__ X, float *__restrict__ TI,
                                                              const float *__restrict__ scale,
                                                              const float *__restrict__ shift, int H, int W, int C,
@@ -175,25 +191,7 @@ __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__rest
     }
     float *dst = TI + static_cast<size_t>(idx) * VEC;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        if (STREAM)
-            stream_store(dst + i * plane, t[i]);
-        else
-            *reinterpret_cast<V *>(dst + i * plane) = t[i];
-    }
-}
-
-// Planes above this size (all 16 together) are written with streaming stores: half of the Infinity
-// Cache, beyond which the consumer cannot expect to find them resident.  SWC_IMTRANS_STREAM=0/1 in the
-// environment forces the choice (read once).
-constexpr size_t kStreamBytes = 128ull << 20;
-bool use_stream_stores(size_t out_bytes)
-{
-    static const int forced = [] {
-        const char *e = std::getenv("SWC_IMTRANS_STREAM");
-        return e == nullptr || e[0] == '\0' ? -1 : (e[0] != '0');
-    }();
-    return forced >= 0 ? forced != 0 : out_bytes > kStreamBytes;
+    for (int i = 0; i < 16; ++i) stream_store(dst + i * plane, t[i]);
 }
 
 template <int VEC, bool RELU, bool AFFINE, typename Idx>
@@ -205,13 +203,10 @@ int launch_direct(const float *X, const float *scale, const float *shift, float 
     const size_t blocks = (items + 255) / 256;
     const dim3 grid(static_cast<unsigned>(blocks)), block(256);
     if (bf16_out)
-        imtrans_direct_kernel<VEC, RELU, AFFINE, false, true, Idx><<<grid, block, 0, stream>>>(
-            X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
-    else if (use_stream_stores(16 * M * C * sizeof(float)))
-        imtrans_direct_kernel<VEC, RELU, AFFINE, true, false, Idx><<<grid, block, 0, stream>>>(
+        imtrans_direct_kernel<VEC, RELU, AFFINE, true, Idx><<<grid, block, 0, stream>>>(
             X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
     else
-        imtrans_direct_kernel<VEC, RELU, AFFINE, false, false, Idx><<<grid, block, 0, stream>>>(
+        imtrans_direct_kernel<VEC, RELU, AFFINE, false, Idx><<<grid, block, 0, stream>>>(
             X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
     return check_launch();
 }

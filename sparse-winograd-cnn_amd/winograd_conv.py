@@ -24,8 +24,8 @@ class WinogradConv(torch.nn.Module):
       it for a rank-3 shape.
     * ``mask``: optional 0/1 array of the weight's shape; the reference multiplies it in on
       every step (:23-25).  Here W*mask is recomputed only while gradients are being recorded
-      (so that they flow to W through the mask); otherwise the product is cached and refreshed
-      by ``refresh()`` after W changes.
+      (so that they flow to W through the mask); otherwise the product is cached until W or
+      mask is written to again (in place or replaced).
 
     W is a trainable parameter; gradients come from ``winograd2x2_conv_grad``.
     """
@@ -49,25 +49,36 @@ class WinogradConv(torch.nn.Module):
         self._bf16 = None
 
     def refresh(self):
-        """Recompute the cached W*mask and its bf16 copy (call after changing W or mask)."""
+        """Drop the cached W*mask and its bf16 copy.  Not needed after in-place updates of W or mask
+        (optimizer steps, ``load_state_dict``): the caches are keyed on the tensors' version counters
+        and storage, so those are noticed by themselves."""
         self._masked = None
         self._bf16 = None
 
+    def _weight_key(self):
+        # In-place writes bump _version; a replaced or moved tensor changes data_ptr / device.
+        w, m = self.W, self.mask
+        return (w._version, w.data_ptr(), w.device, None if m is None else (m._version, m.data_ptr()))
+
     def bf16_weight(self):
         """W*mask as the [16,K,C] bfloat16 tensor the bf16-stored kernel reads; cached like masked_weight()."""
-        w = self.masked_weight()
-        cached = getattr(self, "_bf16", None)
-        if cached is None or cached[0] is not w or cached[1] != w._version or cached[2].device != w.device:
-            cached = (w, w._version, winograd2x2_conv.winograd2x2_conv.winograd2x2_weights_bf16(w))
+        key = self._weight_key()
+        cached = self._bf16
+        if cached is None or cached[0] != key:
+            cached = (key, winograd2x2_conv.winograd2x2_conv.winograd2x2_weights_bf16(self.masked_weight()))
             self._bf16 = cached
-        return cached[2]
+        return cached[1]
 
     def masked_weight(self):
+        """W*mask without autograd history, recomputed only when W or mask changed since the last call."""
         if self.mask is None:
             return self.W.data
-        if self._masked is None or self._masked.device != self.W.device:
-            self._masked = (self.W.data * self.mask).contiguous()
-        return self._masked
+        key = self._weight_key()
+        cached = self._masked
+        if cached is None or cached[0] != key:
+            cached = (key, (self.W.data * self.mask).contiguous())
+            self._masked = cached
+        return cached[1]
 
     def forward(self, x, affine=None, residual=None):
         """``affine=(scale, shift)`` and ``residual`` (forward only) are applied to the result inside

@@ -144,6 +144,37 @@ def test_layer_wrappers_signatures():
         WinogradImTrans(torch.zeros(1, 4, 4, 4), nl=3)
 
 
+def test_masked_weight_cache_follows_weight_updates():
+    """The cached W*mask must not outlive an in-place change of W or mask (optimizer step,
+    load_state_dict), and an unmasked layer must hand out W itself."""
+    from winograd_conv import WinogradConv
+    mask = np.zeros((16, 4, 6), dtype=np.float32)
+    mask[:, :, ::2] = 1
+    m = torch.from_numpy(mask)
+    layer = WinogradConv(4, 6, mask=mask, W_init=lambda w: w.fill_(2.0))
+    first = layer.masked_weight()
+    assert torch.equal(first, m * 2.0)
+    assert layer.masked_weight() is first                      # unchanged weights: cache hit
+    opt = torch.optim.SGD(layer.parameters(), lr=0.5)
+    layer.W.grad = torch.ones_like(layer.W)
+    opt.step()                                                 # W <- 1.5, in place
+    assert torch.equal(layer.masked_weight(), m * 1.5)
+    state = {k: v.clone() for k, v in layer.state_dict().items()}
+    state["W"].fill_(-3.0)
+    layer.load_state_dict(state)
+    assert torch.equal(layer.masked_weight(), m * -3.0)
+    with torch.no_grad():
+        layer.mask.zero_()                                     # the mask changes too
+    assert torch.count_nonzero(layer.masked_weight()) == 0
+    plain = WinogradConv(4, 6)
+    assert plain.masked_weight().data_ptr() == plain.W.data_ptr()
+    k1 = plain._weight_key()
+    assert plain._weight_key() == k1                           # stable key: the bf16 copy is reused
+    with torch.no_grad():
+        plain.W.mul_(2.0)
+    assert plain._weight_key() != k1
+
+
 def test_weight_preparation_matches_oracle(oracle):
     from winograd_weights import gen_prune_mask, kernel_transform
     rng = np.random.default_rng(0)
