@@ -345,6 +345,26 @@ def main():
             print("bench.py: HIP graph capture failed (%s); eager timing only" % e, file=sys.stderr)
             ms_step_graph = None
 
+    # The same step through the Python surface the reference's callers use (winograd2x2_imTrans(...) and
+    # winograd2x2_conv(...), ResNet-18-var/winograd_imtrans.py:16-17, winograd_conv.py:28): shape checks, output
+    # allocation and one C call per op on every call.
+    if stored:
+        def py_step():
+            return winograd2x2_conv(winograd2x2_imTrans(x, relu=True, out_dtype=torch.bfloat16), w16)
+    else:
+        def py_step():
+            return winograd2x2_conv(winograd2x2_imTrans(x, relu=True), w, precision=args.precision)
+    for _ in range(args.warmup):
+        py_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        py_step()
+    t_host = time.perf_counter() - t0
+    torch.cuda.synchronize()
+    ms_step_python = (time.perf_counter() - t0) * 1e3 / args.steps
+    us_host_python = t_host * 1e6 / args.steps   # host time per step alone (the launches are asynchronous)
+
     # Per-kernel average launch durations, HIP events on the launching (current) stream.
     ms_imtrans = time_loop(f_imtrans, args.steps, torch)
     ms_conv = time_loop(f_conv, args.steps, torch)
@@ -432,6 +452,8 @@ def main():
         "launch": "hip graph replay of the K steps" if ms_best != ms_step else "eager",
         "ms_per_step_eager": round(ms_step, 5),
         "ms_per_step_graph": None if ms_step_graph is None else round(ms_step_graph, 5),
+        "ms_per_step_python_ops": round(ms_step_python, 5),
+        "python_ops_host_us_per_step": round(us_host_python, 1),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

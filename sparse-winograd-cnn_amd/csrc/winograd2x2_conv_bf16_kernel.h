@@ -137,6 +137,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
         // issued after it are outstanding; after the barrier every wave has also finished reading the
         // slot that the next copies overwrite (it was fetched one step earlier still).
         if (!(ABL & 2)) wait_vmcnt<(NSTAGE - 2) * Cfg::COPIES>();
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's own reads of the slot about to be refilled are done
         if (!(ABL & 1)) __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (!(ABL & 4)) issue();

@@ -467,7 +467,8 @@ __device__ __forceinline__ void async_copy16(const float *base, unsigned voff, u
         "global_load_lds_dwordx4 %0, %1"
         :
         : "v"(voff), "s"(base), "s"(lds_base)
-        : "memory");  // m0 is a reserved register: the compiler never keeps a value in it across statements
+        : "memory");  // m0 cannot be named as a clobber: the compiler treats it as reserved (-Winline-asm) and
+                      // itself rewrites it immediately before each of its own instructions that read it
 }
 
 // s_waitcnt with only the vector-memory counter constrained (gfx9 encoding: vmcnt in bits 3:0

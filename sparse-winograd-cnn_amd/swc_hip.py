@@ -115,6 +115,31 @@ def dims(shape):
     return (ctypes.c_int64 * len(shape))(*[int(s) for s in shape])
 
 
+class on_device(object):
+    """``with on_device(dev) as stream:`` makes ``dev`` the current HIP device if it is not already (the
+    usual case costs one query instead of a device switch and back) and yields the raw handle of
+    PyTorch's current stream on it."""
+    __slots__ = ("dev", "ctx")
+
+    def __init__(self, dev):
+        self.dev = dev
+        self.ctx = None
+
+    def __enter__(self):
+        import torch
+
+        idx = self.dev.index
+        if idx is not None and idx != torch.cuda.current_device():
+            self.ctx = torch.cuda.device(self.dev)
+            self.ctx.__enter__()
+        return torch.cuda.current_stream().cuda_stream
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
+
+
 def check(status, where):
     if status != SWC_OK:
         raise SwcError(status, where)

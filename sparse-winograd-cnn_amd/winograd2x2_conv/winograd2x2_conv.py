@@ -18,10 +18,28 @@ PRECISIONS = {"fp32": 0, "bf16": 1}
 
 def winograd2x2_conv_shape(i_shape, w_shape):
     """I [16,B,nH,nW,C], W [16,C,K] -> [B,2nH,2nW,K] (winograd2x2_conv.py:19-29), computed by the C++ host wrapper."""
-    out = swc_hip.dims([0] * 4)
-    swc_hip.check(swc_hip.lib().swc_winograd2x2_conv_op_shape(
-        len(i_shape), swc_hip.dims(i_shape), len(w_shape), swc_hip.dims(w_shape), out), "winograd2x2_conv")
-    return tuple(out)
+    return _plan(tuple(i_shape), tuple(w_shape))[0]
+
+
+# (I.shape, W.shape) -> (output shape, and the three dimension arrays swc_winograd2x2_conv_op_compute takes): shapes
+# are validated by the C++ host wrapper once; a layer that is called again with the same shapes pays one lookup.
+_PLANS = {}
+
+
+def _plan(i_shape, w_shape):
+    key = (i_shape, w_shape)
+    plan = _PLANS.get(key)
+    if plan is None:
+        out = swc_hip.dims([0] * 4)
+        i_dims, w_dims = swc_hip.dims(i_shape), swc_hip.dims(w_shape)
+        swc_hip.check(swc_hip.lib().swc_winograd2x2_conv_op_shape(len(i_shape), i_dims, len(w_shape), w_dims, out),
+                      "winograd2x2_conv")
+        shape = tuple(out)
+        plan = (shape, i_dims, w_dims, swc_hip.dims(shape))
+        if len(_PLANS) >= 1024:
+            _PLANS.clear()
+        _PLANS[key] = plan
+    return plan
 
 
 def _forward(I, W, precision, out, scale=None, shift=None, residual=None):
@@ -31,11 +49,11 @@ def _forward(I, W, precision, out, scale=None, shift=None, residual=None):
     W = swc_hip.require_cuda_f32(W, "W", 3)
     if W.device != I.device:
         raise ValueError("I and W must be on the same device")
-    shape = winograd2x2_conv_shape(I.shape, W.shape)
+    shape, i_dims, w_dims, o_dims = _plan(I.shape, W.shape)
     if out is None:
         out = torch.empty(shape, dtype=torch.float32, device=I.device)
     else:
-        if tuple(out.shape) != shape or out.dtype != torch.float32 or out.device != I.device or not out.is_contiguous():
+        if out.shape != shape or out.dtype != torch.float32 or out.device != I.device or not out.is_contiguous():
             raise ValueError("out must be a contiguous float32 tensor of shape %s on %s" % (shape, I.device))
     if (scale is None) != (shift is None):
         raise ValueError("scale and shift go together")
@@ -49,8 +67,7 @@ def _forward(I, W, precision, out, scale=None, shift=None, residual=None):
         residual = swc_hip.require_cuda_f32(residual, "residual", 4)
         if tuple(residual.shape) != shape:
             raise ValueError("residual must have the output's shape %s" % (shape,))
-    with torch.cuda.device(I.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with swc_hip.on_device(I.device) as stream:
         if epilogue:
             _, B, nH, nW, C = I.shape
             st = swc_hip.lib().swc_winograd2x2_conv_epilogue(
@@ -59,8 +76,8 @@ def _forward(I, W, precision, out, scale=None, shift=None, residual=None):
                 C, B, nH, nW, shape[3], 1, 1, PRECISIONS[precision], stream)
         else:
             st = swc_hip.lib().swc_winograd2x2_conv_op_compute(
-                I.data_ptr(), 5, swc_hip.dims(I.shape), W.data_ptr(), 3, swc_hip.dims(W.shape),
-                out.data_ptr(), 4, swc_hip.dims(out.shape), PRECISIONS[precision], stream)
+                I.data_ptr(), 5, i_dims, W.data_ptr(), 3, w_dims, out.data_ptr(), 4, o_dims, PRECISIONS[precision],
+                stream)
     swc_hip.check(st, "winograd2x2_conv")
     return out
 
@@ -72,9 +89,8 @@ def winograd2x2_weights_bf16(W):
     if W.shape[0] != 16:
         raise ValueError("W must have shape [16,C,K]")
     out = torch.empty((16, W.shape[2], W.shape[1]), dtype=torch.bfloat16, device=W.device)
-    with torch.cuda.device(W.device):
-        st = swc_hip.lib().swc_winograd2x2_weights_bf16(W.data_ptr(), out.data_ptr(), W.shape[1], W.shape[2],
-                                                        torch.cuda.current_stream().cuda_stream)
+    with swc_hip.on_device(W.device) as stream:
+        st = swc_hip.lib().swc_winograd2x2_weights_bf16(W.data_ptr(), out.data_ptr(), W.shape[1], W.shape[2], stream)
     swc_hip.check(st, "winograd2x2_weights_bf16")
     return out
 
@@ -94,7 +110,7 @@ def _forward_bf16_stored(I, W, out, scale, shift, residual):
     shape = (B, 2 * nH, 2 * nW, K)
     if out is None:
         out = torch.empty(shape, dtype=torch.float32, device=I.device)
-    elif tuple(out.shape) != shape or out.dtype != torch.float32 or out.device != I.device or not out.is_contiguous():
+    elif out.shape != shape or out.dtype != torch.float32 or out.device != I.device or not out.is_contiguous():
         raise ValueError("out must be a contiguous float32 tensor of shape %s on %s" % (shape, I.device))
     if (scale is None) != (shift is None):
         raise ValueError("scale and shift go together")
@@ -107,11 +123,11 @@ def _forward_bf16_stored(I, W, out, scale, shift, residual):
         residual = swc_hip.require_cuda_f32(residual, "residual", 4)
         if tuple(residual.shape) != shape:
             raise ValueError("residual must have the output's shape %s" % (shape,))
-    with torch.cuda.device(I.device):
+    with swc_hip.on_device(I.device) as stream:
         st = swc_hip.lib().swc_winograd2x2_conv_bf16in(
             I.data_ptr(), W.data_ptr(), out.data_ptr(), None if scale is None else scale.data_ptr(),
             None if shift is None else shift.data_ptr(), None if residual is None else residual.data_ptr(),
-            C, B, nH, nW, K, 1, 1, torch.cuda.current_stream().cuda_stream)
+            C, B, nH, nW, K, 1, 1, stream)
     swc_hip.check(st, "winograd2x2_conv (bf16-stored operands)")
     return out
 
@@ -129,10 +145,10 @@ def winograd2x2_conv_grad(i1, i2, grad):
     K = W.shape[2]
     dI, dW = torch.empty_like(I), torch.empty_like(W)
     tmp = torch.empty(16 * B * nH * nW * K, dtype=torch.float32, device=I.device)  # as winograd2x2_conv_grad_op.cc:69-71
-    with torch.cuda.device(I.device):
+    with swc_hip.on_device(I.device) as stream:
         st = swc_hip.lib().swc_winograd2x2_conv_grad(
             I.data_ptr(), W.data_ptr(), grad.data_ptr(), dI.data_ptr(), dW.data_ptr(), tmp.data_ptr(), None,
-            C, B, 2 * nH, 2 * nW, K, 1, 1, torch.cuda.current_stream().cuda_stream)
+            C, B, 2 * nH, 2 * nW, K, 1, 1, stream)
     swc_hip.check(st, "winograd2x2_conv_grad")
     return dI, dW
 
@@ -173,7 +189,9 @@ def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, r
         return _forward_bf16_stored(I, W, out, scale, shift, residual)
     if (scale is not None or residual is not None) and needs_grad:
         raise NotImplementedError("the scale/shift/residual epilogue is forward only")
-    if out is None and needs_grad:
+    if needs_grad:
+        if out is not None:
+            raise NotImplementedError("out= is forward only: the result written there would carry no gradient")
         return _ConvFunction.apply(I, W, precision)
     return _forward(I, W, precision, out, scale, shift, residual)
 

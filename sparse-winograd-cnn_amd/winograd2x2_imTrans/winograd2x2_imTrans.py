@@ -16,15 +16,31 @@ import swc_hip  # noqa: E402
 
 def winograd2x2_imTrans_shape(shape):
     """[B,H,W,C] -> [16,B,(H+1)/2,(W+1)/2,C] (winograd2x2_imTrans.py:20-27), computed by the C++ host wrapper."""
-    out = swc_hip.dims([0] * 5)
-    swc_hip.check(swc_hip.lib().swc_winograd2x2_imtrans_op_shape(len(shape), swc_hip.dims(shape), out),
-                  "winograd2x2_imTrans")
-    return tuple(out)
+    return _plan(tuple(shape))[0]
+
+
+# I.shape -> (output shape, and the two dimension arrays swc_winograd2x2_imtrans_op_compute takes): validated by the
+# C++ host wrapper once per shape.
+_PLANS = {}
+
+
+def _plan(shape):
+    plan = _PLANS.get(shape)
+    if plan is None:
+        out = swc_hip.dims([0] * 5)
+        i_dims = swc_hip.dims(shape)
+        swc_hip.check(swc_hip.lib().swc_winograd2x2_imtrans_op_shape(len(shape), i_dims, out), "winograd2x2_imTrans")
+        o_shape = tuple(out)
+        plan = (o_shape, i_dims, swc_hip.dims(o_shape))
+        if len(_PLANS) >= 1024:
+            _PLANS.clear()
+        _PLANS[shape] = plan
+    return plan
 
 
 def _forward(I, relu, out, scale=None, shift=None, out_dtype=torch.float32):
     I = swc_hip.require_cuda_f32(I, "I", 4)
-    shape = winograd2x2_imTrans_shape(I.shape)
+    shape, i_dims, o_dims = _plan(I.shape)
     if (scale is None) != (shift is None):
         raise ValueError("scale and shift go together")
     if scale is not None:
@@ -37,10 +53,9 @@ def _forward(I, relu, out, scale=None, shift=None, out_dtype=torch.float32):
     if out is None:
         out = torch.empty(shape, dtype=out_dtype, device=I.device)
     else:
-        if tuple(out.shape) != shape or out.dtype != out_dtype or out.device != I.device or not out.is_contiguous():
+        if out.shape != shape or out.dtype != out_dtype or out.device != I.device or not out.is_contiguous():
             raise ValueError("out must be a contiguous %s tensor of shape %s on %s" % (out_dtype, shape, I.device))
-    with torch.cuda.device(I.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with swc_hip.on_device(I.device) as stream:
         if out_dtype == torch.bfloat16:
             B, H, W, C = I.shape
             st = swc_hip.lib().swc_winograd2x2_imtrans_bf16out(
@@ -52,9 +67,8 @@ def _forward(I, relu, out, scale=None, shift=None, out_dtype=torch.float32):
                 I.data_ptr(), scale.data_ptr(), shift.data_ptr(), out.data_ptr(), C, B, H, W, 1, 1, int(bool(relu)),
                 stream)
         else:
-            st = swc_hip.lib().swc_winograd2x2_imtrans_op_compute(
-                I.data_ptr(), 4, swc_hip.dims(I.shape), out.data_ptr(), 5, swc_hip.dims(out.shape), int(bool(relu)),
-                stream)
+            st = swc_hip.lib().swc_winograd2x2_imtrans_op_compute(I.data_ptr(), 4, i_dims, out.data_ptr(), 5, o_dims,
+                                                                  int(bool(relu)), stream)
     swc_hip.check(st, "winograd2x2_imTrans")
     return out
 
@@ -93,8 +107,7 @@ def winograd2x2_imTrans_grad(grad, H=None, W=None, relu_output=None, relu_input=
             raise ValueError("relu_output must have grad's shape")
         mask_ptr = relu_output.data_ptr()
     out = torch.empty((B, H, W, C), dtype=torch.float32, device=grad.device)
-    with torch.cuda.device(grad.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with swc_hip.on_device(grad.device) as stream:
         if relu_input is not None:
             st = swc_hip.lib().swc_winograd2x2_imtrans_grad_relu_input(grad.data_ptr(), relu_input.data_ptr(),
                                                                        out.data_ptr(), C, B, H, W, 1, 1, stream)
@@ -134,12 +147,14 @@ def winograd2x2_imTrans(I, relu=False, out=None, scale=None, shift=None, out_dty
 
     ``relu=True`` applies the Winograd-domain ReLU inside the same kernel (what
     ``nl(winograd2x2_imTrans(x))`` with ``nl=tf.nn.relu`` computes in
-    ResNet-18-var/winograd_imtrans.py:16-17).  ``out`` may supply the result tensor (forward only).
+    ResNet-18-var/winograd_imtrans.py:16-17).  ``out`` may supply the result tensor (forward only: with an input that requires grad it raises).
     Differentiable: gradients flow through ``winograd2x2_imTrans_grad``.
     """
     needs_grad = isinstance(I, torch.Tensor) and I.requires_grad and torch.is_grad_enabled()
     if (scale is not None or out_dtype != torch.float32) and needs_grad:
         raise NotImplementedError("the scale/shift and bf16-output variants are forward only")
-    if out is None and needs_grad:
+    if needs_grad:
+        if out is not None:
+            raise NotImplementedError("out= is forward only: the result written there would carry no gradient")
         return _ImTransFunction.apply(I, relu)
     return _forward(I, relu, out, scale, shift, out_dtype)

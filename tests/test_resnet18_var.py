@@ -28,9 +28,24 @@ def test_same_padding_rule():
     assert resnet18_var._same_pad(torch.zeros(1, 1, 7, 9), 3, 2) == [1, 1, 1, 1]
 
 
+PRECISIONS = [("fp32", 1e-3), ("bf16", 5e-2), ("bf16_stored", 5e-2)]
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("precision,tol", [("fp32", 1e-3), ("bf16", 5e-2), ("bf16_stored", 5e-2)])
+@pytest.mark.parametrize("precision,tol", PRECISIONS)
 def test_forward_matches_oracle_path(oracle, precision, tol):
+    _forward_against_oracle_path(oracle, precision, tol, batch=2, size=64, check_unfolded=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("precision,tol", PRECISIONS)
+def test_forward_matches_oracle_path_at_224(oracle, precision, tol):
+    # Benchmark config 5's image size: the 16 layers run at 56/28/14/14 as in
+    # imagenet-resnet-transWino-prune.py:113-212 (the 64x64 case above runs them at 16/8/4/4).
+    _forward_against_oracle_path(oracle, precision, tol, batch=2, size=224, check_unfolded=False)
+
+
+def _forward_against_oracle_path(oracle, precision, tol, batch, size, check_unfolded):
     # Same module, same weights: once on the GPU through the HIP ops, once on the CPU with the two
     # Winograd ops replaced by the oracle.
     import resnet18_var
@@ -47,7 +62,7 @@ def test_forward_matches_oracle_path(oracle, precision, tol):
         bn.running_var.uniform_(0.5, 1.5)
         bn.weight.data.uniform_(0.5, 1.5)
         bn.bias.data.normal_(0, 0.1)
-    image = torch.from_numpy(rng.standard_normal((2, 64, 64, 3)).astype(np.float32))
+    image = torch.from_numpy(rng.standard_normal((batch, size, size, 3)).astype(np.float32))
 
     def cpu_imtrans(x, nl=None, affine=None, out_dtype=torch.float32):
         x = x.numpy()
@@ -79,9 +94,11 @@ def test_forward_matches_oracle_path(oracle, precision, tol):
     for c in model.winograd_convs():
         c.refresh()
     got = model(image.to(dev)).cpu().numpy()
-    assert got.shape == want.shape == (2, 1000)
+    assert got.shape == want.shape == (batch, 1000)
     assert np.isfinite(got).all()
     assert rel_max(got, want) <= tol
+    if not check_unfolded:
+        return
     # Folding the BatchNorm into the transform changes roundings only (one fma per pixel instead of
     # PyTorch's normalisation arithmetic).
     unfolded = resnet18_var.ResNet18Var(masks=masks, precision=precision, fold_bn=False)
@@ -90,3 +107,48 @@ def test_forward_matches_oracle_path(oracle, precision, tol):
     for c in unfolded.winograd_convs():
         c.refresh()
     assert rel_max(unfolded(image.to(dev)).cpu().numpy(), got) <= tol
+
+
+# The distinct (H = W, C, K) of the 16 layers (imagenet-resnet-transWino-prune.py:117-211): 4x (56,64,64), (28,64,128),
+# 3x (28,128,128), (14,128,256), 3x (14,256,256), (14,256,512), 3x (14,512,512).
+LAYER_SHAPES = [(56, 64, 64), (28, 64, 128), (28, 128, 128), (14, 128, 256), (14, 256, 256), (14, 256, 512), (14, 512, 512)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("precision", ["fp32", "bf16", "bf16_stored"])
+@pytest.mark.parametrize("hw,C,K", LAYER_SHAPES)
+def test_layers_at_batch_128(oracle, hw, C, K, precision):
+    """Every layer shape of config 5 at its real batch (N = 128), so that the launcher makes the choice it
+    makes in the benchmark: the transform is compared bit for bit and the convolution within tolerance with
+    the oracle on the first and the last two images (tiles are independent, so a slice of the batch has the
+    values it would have alone; the last images sit in the ragged final row groups)."""
+    import swc_hip
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv
+    from winograd2x2_imTrans.winograd2x2_imTrans import winograd2x2_imTrans
+    dev = torch.device("cuda:0")
+    N, k = 128, 2
+    gen = torch.Generator(device=dev).manual_seed(hw * 1000 + C + K)
+    x = torch.randn((N, hw, hw, C), device=dev, generator=gen)
+    w = (np.random.default_rng(C * K).standard_normal((16, C, K)) * 0.05).astype(np.float32)
+    oracle.gen_prune_mask(w, 0.2)
+    w_gpu = torch.from_numpy(w).to(dev)
+    stored = precision == "bf16_stored"
+    ti = winograd2x2_imTrans(x, relu=True, out_dtype=torch.bfloat16 if stored else torch.float32)
+    y = winograd2x2_conv(ti, w_gpu, precision="fp32" if stored else precision)
+    kernel = swc_hip.lib().swc_winograd2x2_conv_last_kernel().decode()
+    assert y.shape == (N, hw, hw, K)
+    for sl in (slice(0, k), slice(N - k, N)):
+        x_cpu = x[sl].cpu().numpy()
+        ti_want = oracle.imtrans(x_cpu, relu=True)
+        if stored:
+            assert np.array_equal(ti[:, sl].view(torch.int16).cpu().numpy().view(np.uint16), oracle.bf16_bits(ti_want))
+            ti_want, w_want = oracle.round_bf16(ti_want), oracle.round_bf16(w)
+        else:
+            assert np.array_equal(ti[:, sl].cpu().numpy(), ti_want)
+            w_want = w
+            if precision == "bf16":
+                ti_want, w_want = oracle.round_bf16(ti_want), oracle.round_bf16(w)
+        want = oracle.conv(ti_want, w_want, acc64=True)
+        assert rel_max(y[sl].cpu().numpy(), want) <= 1e-4, (kernel, sl)
+    if precision == "fp32":
+        assert kernel != "sync", kernel   # every model shape runs on one of the copy-ring tilings
