@@ -2,9 +2,10 @@
  * C ABI of the MI355X (gfx950) Winograd F(2x2,3x3) forward ops.
  *
  * Plain pointers and sizes only.  Every device pointer is owned by the caller; no
- * entry point allocates or frees device memory, keeps state between calls, or
- * synchronises: work is queued on `stream` (a hipStream_t passed as void*; NULL is
- * the null stream) and the call returns.  Calls are re-entrant and thread-safe.
+ * entry point allocates or frees device memory or synchronises: work is queued on
+ * `stream` (a hipStream_t passed as void*; NULL is the null stream) and the call
+ * returns.  Calls are re-entrant and thread-safe, and keep no state between calls
+ * (the one exception says so: swc_winograd2x2_conv_force_tiling sets a per-thread choice).
  *
  * Citations name the interface of the reference (xingyul/sparse-winograd-cnn) that
  * each entry point stands in for; paths are relative to the reference checkout.
@@ -43,6 +44,12 @@ SWC_API const char *swc_version(void);
  * groups of up to 112 / 32 rows, dealt evenly over the CUs).  Which one runs depends only on the shapes
  * and pointer alignment; all give the same results to within the order of the reduction over C. */
 SWC_API const char *swc_winograd2x2_conv_last_kernel(void);
+/* Diagnostic with no counterpart in the reference, for benchmarks and tests that compare the tilings: makes
+ * the calling thread's later swc_winograd2x2_conv calls (and the data-gradient GEMM of swc_winograd2x2_conv_grad)
+ * use the named kernel ("ring32", "ring16", "tall16", "short16", "sync") where the shapes allow it and "sync"
+ * where they do not; NULL or "" gives the choice back to the launcher.  Returns SWC_ERR_UNSUPPORTED for an
+ * unknown name. */
+SWC_API int swc_winograd2x2_conv_force_tiling(const char *name);
 
 /* ---------------------------------------------------------------------------
  * Launcher level: what the reference's TensorFlow op kernels call.
@@ -240,10 +247,7 @@ SWC_API int swc_winograd2x2_relu_conv_bf16(const float *Input, const float *InSc
  * tmp_data_buffer must hold 16*B*nH*nW*K floats (the caller's temporary, as at
  * winograd2x2_conv_grad_op.cc:69-71); tmp_ptr_buffer is ignored.  TInput_grad is also used as
  * scratch (partial sums of Weight_grad) before it receives its result, so it must not alias an input.
- * The TInput_grad GEMM runs in rocBLAS (as does the Weight_grad GEMM for shapes the library's own
- * kernel does not take: M % 32, C % 4, K % 4, alignment); the first call on a host thread creates
- * that thread's rocBLAS handle, which is the one piece of state (and device memory) this library
- * ever owns.
+ * Both GEMMs of the reference (:103-108, :115-120) run on this library's own kernels.
  */
 SWC_API int swc_winograd2x2_conv_grad(const float *TInput, const float *Weight, const float *Output_grad,
                                       float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,

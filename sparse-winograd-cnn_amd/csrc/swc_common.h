@@ -13,6 +13,9 @@ int note_hip_error(hipError_t e);
 // Records which convolution kernel a call chose, for swc_winograd2x2_conv_last_kernel().
 void note_conv_kernel(const char *name);
 
+// The tiling set with swc_winograd2x2_conv_force_tiling() on this host thread, or nullptr.
+const char *forced_conv_tiling();
+
 inline int check_launch()
 {
     hipError_t e = hipGetLastError();

@@ -1,11 +1,17 @@
 // Status strings, version and the per-thread record of the last HIP error.
+#include <cstring>
+#include <initializer_list>
+
 #include "swc_common.h"
 
 namespace swc {
 namespace {
 thread_local int g_last_hip_error = 0;
 thread_local const char *g_conv_kernel = "";
+thread_local char g_forced_tiling[16] = "";
 }
+
+const char *forced_conv_tiling() { return g_forced_tiling[0] != '\0' ? g_forced_tiling : nullptr; }
 
 void note_conv_kernel(const char *name) { g_conv_kernel = name; }
 
@@ -33,5 +39,20 @@ extern "C" const char *swc_strerror(int status)
 extern "C" int swc_last_hip_error(void) { return swc::g_last_hip_error; }
 
 extern "C" const char *swc_winograd2x2_conv_last_kernel(void) { return swc::g_conv_kernel; }
+
+extern "C" int swc_winograd2x2_conv_force_tiling(const char *name)
+{
+    if (name == nullptr || name[0] == '\0') {
+        swc::g_forced_tiling[0] = '\0';
+        return SWC_OK;
+    }
+    for (const char *known : {"sync", "ring32", "ring16", "tall16", "short16"}) {
+        if (std::strcmp(name, known) == 0) {
+            std::strcpy(swc::g_forced_tiling, known);
+            return SWC_OK;
+        }
+    }
+    return SWC_ERR_UNSUPPORTED;
+}
 
 extern "C" const char *swc_version(void) { return "0.1"; }

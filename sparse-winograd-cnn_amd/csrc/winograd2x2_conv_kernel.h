@@ -481,65 +481,69 @@ __device__ __forceinline__ void wait_vmcnt()
     asm volatile("" ::: "memory");
 }
 
-// Dynamic LDS the async kernel needs at launch: NSTAGE ring slots of one A and one B tile (the B
+// What the ring kernel does with the finished product tile P_i of a position:
+//   RING_FORWARD: folds it into the four output tiles (Y_j +-= P_i) and stores Out [B,2nH,2nW,N] at the end; the B
+//                 operand is Wt [16][R][N] (reduction index slow), as the forward weights are.
+//   RING_DGRAD:   stores it as plane i of Out [16][M][N]; the B operand is Wt [16][N][R] (reduction index fast):
+//                 with A = dP, R = K, N = C and Wt = W this is dTI_i = dP_i . W_i^T, the first GEMM of the
+//                 reference's backward pass (winograd2x2_conv_grad_cuda.cu.cc:103-108).
+enum RingMode { RING_FORWARD = 0, RING_DGRAD = 1 };
+
+// Dynamic LDS the ring kernel needs at launch: NSTAGE ring slots of one A and one B tile (the forward B
 // tile padded by 64 bytes per KiB with 16x16 MFMAs).  Above 64 KiB the launcher must first raise
 // hipFuncAttributeMaxDynamicSharedMemorySize.
-template <typename Cfg, int NSTAGE>
+template <typename Cfg, int NSTAGE, int MODE = RING_FORWARD>
 constexpr int async_lds_bytes()
 {
-    constexpr int nbw = Cfg::BK * Cfg::BN / 4 / 64, bpad = Cfg::BPAD;
+    constexpr int nbw = Cfg::BK * Cfg::BN / 4 / 64, bpad = MODE == RING_FORWARD ? Cfg::BPAD : 0;
     return NSTAGE * (Cfg::BM * Cfg::BK + Cfg::BK * Cfg::BN + nbw * bpad) * 4;
 }
 
-// BF16: the operands are rounded to bf16 (round-to-nearest-even, v_cvt_pk_bf16_f32) after they are read
-// from LDS and multiplied with v_mfma_f32_32x32x16_bf16; accumulation, fold and stores stay fp32.
-// ABL: timing ablations for kernel development (bit 0: no barrier, 1: no copy wait, 2: no copies,
-// 3: no LDS reads, 4: no output stores, 5: fold only the last position); results are wrong with any bit set.  Always 0 in the library.
-template <typename Cfg, int NSTAGE, bool BF16 = false, int ABL = 0>
-__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_mfma_async_kernel(
-    const float *__restrict__ TI, const float *__restrict__ Wt, float *__restrict__ Out, size_t M, int C, int K, int nH,
-    int nW, unsigned tiles_n, unsigned rows_per_wg, ConvEpilogue ep)
+// The ring kernel's body.  A [16][M][R] row-major (R = reduction length, a multiple of BK), the workgroup's tile
+// starts at row m0, column n0 and owns rows_valid <= BM rows; wave tile at (wm0, wn0) within it; N = number of
+// output columns.
+// BF16 (forward only): the operands are rounded to bf16 (round-to-nearest-even, v_cvt_pk_bf16_f32) after they are
+// read from LDS and multiplied with v_mfma_f32_32x32x16_bf16; accumulation, fold and stores stay fp32.
+template <typename Cfg, int NSTAGE, bool BF16, int MODE>
+__device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, const float *__restrict__ Wt,
+                                               float *__restrict__ Out, size_t M, int R, int N, int nW, const size_t m0,
+                                               const int n0, const unsigned rows_valid, const int wm0, const int wn0,
+                                               const ConvEpilogue ep)
 {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT, MF = Cfg::MF, LG = Cfg::LG, KG = Cfg::KG;
     constexpr int TM = Cfg::TM, TN = Cfg::TN;
     constexpr int KS = BK / KG, CH = BK / 4, NWAVES = NT / 64;
+    constexpr bool DGRAD = MODE == RING_DGRAD;
     // Copies are wave-wide: 64 lanes x 16 bytes = 1 KiB.  NAW / NBW of them make an A / B tile; every
     // wave issues the same number (NA + NB) per step so that all waves count outstanding copies alike;
     // where the tile does not divide evenly the surplus copies repeat an earlier one (same bytes twice).
     constexpr int NAW = BM * CH / 64, NBW = BK * BN / 4 / 64;
     constexpr int NA = (NAW + NWAVES - 1) / NWAVES, NB = (NBW + NWAVES - 1) / NWAVES;
-    // With 16x16 MFMAs the four lane groups of a B operand read hit rows 4 apart; 64 bytes of padding
-    // after every copy (4 rows of 64 floats) put them on different banks.
-    constexpr int BPAD = Cfg::BPAD;  // floats
+    // Forward B tile with 16x16 MFMAs: the four lane groups of an operand read hit rows 4 apart; 64 bytes of
+    // padding after every copy (4 rows of 64 floats) put them on different banks.
+    constexpr int BPAD = DGRAD ? 0 : Cfg::BPAD;  // floats
     static_assert(BPAD == 0 || BN == 64, "the padded B layout assumes one copy = 4 rows");
     constexpr int A_FLOATS = BM * BK, B_FLOATS = BK * BN + NBW * BPAD, STAGE_FLOATS = A_FLOATS + B_FLOATS;
     constexpr int LPS = NA + NB;  // copies per thread per step
-    // Scheduling granularity (development knobs): reads/copies are dealt out in groups of GR, fold units in groups of GF.
-    constexpr int GR = ((ABL >> 8) & 15) ? ((ABL >> 8) & 15) : 1, GF = ((ABL >> 12) & 31) ? ((ABL >> 12) & 31) : 1;
     static_assert(NSTAGE >= 2, "a ring needs two slots");
     static_assert(KS % 2 == 0, "the MFMA chain of a step is split in two halves");
-    static_assert(!BF16 || (KS == 4 && MF == 32), "the bf16 MFMA consumes 16 reduction indices: a half of a 32-index step");
+    static_assert(!BF16 || (KS == 4 && MF == 32 && !DGRAD), "the bf16 MFMA consumes 16 reduction indices: a half of a 32-index step");
     static_assert((CH & (CH - 1)) == 0, "swizzle needs a power-of-two chunk count");
     static_assert((BM * CH) % 64 == 0 && (BK * BN / 4) % 64 == 0, "tiles are whole wave-wide copies");
-    static_assert((NSTAGE - 2) * LPS < 64, "vmcnt range");
+    static_assert((NSTAGE - 2) * LPS + (DGRAD ? TM * TN * Cfg::REGS : 0) < 64, "vmcnt range");
+    static_assert(!DGRAD || NSTAGE <= 3, "the wait below allows for the stores of one earlier step");
 
-    static_assert(NSTAGE * STAGE_FLOATS * 4 == async_lds_bytes<Cfg, NSTAGE>(), "launcher and kernel agree on the LDS size");
-    extern __shared__ __attribute__((aligned(1024))) float smem[];  // async_lds_bytes<Cfg, NSTAGE>() bytes
-
-    const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
-    // The workgroup's tile starts at row m0 and is BM rows tall, of which the first rows_valid are
-    // its own (rows_per_wg <= BM lets the launcher split M evenly at 16-row granularity).
-    const size_t m0 = static_cast<size_t>(lid / tiles_n) * rows_per_wg;
-    const int n0 = static_cast<int>(lid % tiles_n) * BN;
-    const unsigned rows_valid = static_cast<unsigned>(M - m0 < rows_per_wg ? M - m0 : rows_per_wg);
+    static_assert(NSTAGE * STAGE_FLOATS * 4 == async_lds_bytes<Cfg, NSTAGE, MODE>(), "launcher and kernel agree on the LDS size");
+    extern __shared__ __attribute__((aligned(1024))) float smem[];  // async_lds_bytes<Cfg, NSTAGE, MODE>() bytes
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int li = lane % MF, lg = lane / MF;
-    const int wm0 = (wave / Cfg::WGN) * Cfg::WM, wn0 = (wave % Cfg::WGN) * Cfg::WN;
 
     // Per-thread byte offsets of the copies (constant over the whole kernel) and the
     // wave-uniform LDS byte offsets, relative to a stage, they land at.
+    // A tile (and the B tile of RING_DGRAD): rows of BK/4 16-byte chunks; chunk j of row r sits in slot
+    // r*(BK/4) + (j ^ (r % (BK/4))).
     unsigned a_voff[NA], b_voff[NB];
     unsigned a_lds[NA], b_lds[NB];  // wave-uniform byte offsets within a stage
     const unsigned wave_u = __builtin_amdgcn_readfirstlane(wave);
@@ -550,40 +554,52 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
         unsigned row = slot / CH;
         const unsigned chunk = (slot % CH) ^ (row % CH);
         row = row < rows_valid ? row : rows_valid - 1;
-        a_voff[q] = (row * static_cast<unsigned>(C) + chunk * 4) * 4u;
+        a_voff[q] = (row * static_cast<unsigned>(R) + chunk * 4) * 4u;
         a_lds[q] = wl * 1024u;
     }
 #pragma unroll
     for (int q = 0; q < NB; ++q) {
         const unsigned wl = (q * NWAVES + wave_u) % NBW;
         const unsigned slot = wl * 64 + lane;
-        const unsigned krow = slot / (BN / 4);
-        unsigned n = n0 + (slot % (BN / 4)) * 4;
-        n = n + 4 <= static_cast<unsigned>(K) ? n : static_cast<unsigned>(K) - 4;
-        b_voff[q] = (krow * static_cast<unsigned>(K) + n) * 4u;
-        b_lds[q] = A_FLOATS * 4 + wl * (1024u + BPAD * 4);
+        if (DGRAD) {   // B tile [BN columns][BK reduction indices], swizzled like A
+            unsigned col = slot / CH;
+            const unsigned chunk = (slot % CH) ^ (col % CH);
+            col = n0 + col < static_cast<unsigned>(N) ? n0 + col : static_cast<unsigned>(N) - 1;
+            b_voff[q] = (col * static_cast<unsigned>(R) + chunk * 4) * 4u;
+            b_lds[q] = A_FLOATS * 4 + wl * 1024u;
+        } else {       // B tile [BK reduction indices][BN columns]
+            const unsigned krow = slot / (BN / 4);
+            unsigned n = n0 + (slot % (BN / 4)) * 4;
+            n = n + 4 <= static_cast<unsigned>(N) ? n : static_cast<unsigned>(N) - 4;
+            b_voff[q] = (krow * static_cast<unsigned>(N) + n) * 4u;
+            b_lds[q] = A_FLOATS * 4 + wl * (1024u + BPAD * 4);
+        }
     }
     const unsigned smem_base = lds_address(smem);
 
-    const int nkc = C / BK;
+    const int nkc = R / BK;
     using Acc = AccT<Cfg>;
-    Acc Y[4][TM][TN];
+    Acc Y[DGRAD ? 1 : 4][DGRAD ? 1 : TM][DGRAD ? 1 : TN];
+    if constexpr (!DGRAD) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
+            for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-            for (int tn = 0; tn < TN; ++tn)
+                for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-                for (int r = 0; r < Cfg::REGS; ++r) Y[j][tm][tn][r] = 0.f;
+                    for (int r = 0; r < Cfg::REGS; ++r) Y[j][tm][tn][r] = 0.f;
+    }
 
     // ---- copy issuer: running pointers to the tiles of the next step to fetch -------------
-    // Tile of (pos, c0): A at TI + (pos*M + m0)*C + c0, B at Wt + (pos*C + c0)*K.  Consecutive
-    // steps advance A by BK floats, plus (M-1)*C when the position wraps, and B by BK*K.
-    const float *a_next = TI + m0 * C;
+    // Tile of (pos, c0): A at TI + (pos*M + m0)*R + c0; B at Wt + (pos*R + c0)*N (forward) or
+    // Wt + pos*N*R + c0 (dgrad; the column offset is in b_voff).  Consecutive steps advance A by BK floats, plus
+    // (M-1)*R when the position wraps, and B by BK*N (forward) or by BK, plus (N-1)*R at the wrap (dgrad).
+    const float *a_next = TI + m0 * R;
     const float *b_next = Wt;
-    const size_t a_wrap = (M - 1) * static_cast<size_t>(C);
-    const size_t b_inc = static_cast<size_t>(BK) * K;
+    const size_t a_wrap = (M - 1) * static_cast<size_t>(R);
+    const size_t b_inc = DGRAD ? static_cast<size_t>(BK) : static_cast<size_t>(BK) * N;
+    const size_t b_wrap = DGRAD ? (static_cast<size_t>(N) - 1) * R : 0;
     int kc_next = 0, pos_next = 0;
     unsigned lds_next = smem_base;  // byte address of the next ring slot
     int slot_next = 0;
@@ -603,9 +619,10 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
         if (++kc_next == nkc) {
             kc_next = 0;
             a_next += a_wrap;
+            b_next += b_wrap;
             if (++pos_next == 16) {
                 pos_next = 0;
-                a_next = TI + m0 * C;
+                a_next = TI + m0 * R;
                 b_next = Wt;
             }
         }
@@ -620,14 +637,16 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     // A step's reduction range BK is consumed in two halves of KH groups of KG indices (8 with
     // 32x32 MFMAs, 16 with 16x16).  Within a group, lane group lg feeds indices 4*lg .. 4*lg+3,
     // one per MFMA (the order in which indices are reduced is free as long as A and B agree), so
-    // A comes as one b128 read per group and B as 4 b32 reads, paired so that they merge into
-    // ds_read2_b32.
+    // A comes as one b128 read per group and the forward B as 4 b32 reads, paired so that they merge into
+    // ds_read2_b32; the dgrad B tile has the reduction index fast like A and is read the same way.
     constexpr int KH = KS / 2;
     struct HalfFrag {
         float4 a[KH][TM];
-        float b[KH][4][TN];
+        float b[DGRAD ? 1 : KH][4][TN];
+        float4 bq[DGRAD ? KH : 1][TN];
     };
-    constexpr int NU = KH * (TM + 2 * TN);   // read units per half: KH*TM b128 + KH*2*TN b32 pairs
+    constexpr int NUB = DGRAD ? TN : 2 * TN;    // B read units per group: b128 reads, or b32 pairs
+    constexpr int NU = KH * (TM + NUB);         // read units per half
     // MFMAs per half: fp32 32x32x2 reduces 2 indices each, bf16 32x32x16 all 16 of a half at once.
     constexpr int NM = BF16 ? TM * TN : KH * 4 * TM * TN;
 
@@ -640,16 +659,28 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
             const int row = wm0 + tm * MF + li;
             a_off[k8][tm] = row * CH + ((LG * k8 + lg) ^ (row % CH));  // in 16-byte units
         }
-    // B row k sits at k*BN floats plus BPAD per 4 rows; lane group lg reads rows 4*lg + t of a group.
+    // Forward: B row k sits at k*BN floats plus BPAD per 4 rows; lane group lg reads rows 4*lg + t of a group.
     constexpr int BROW4 = 4 * BN + BPAD;
     const int b_off = A_FLOATS + lg * BROW4 + wn0 + li;
+    int bq_off[DGRAD ? KS : 1][DGRAD ? TN : 1];  // dgrad: 16-byte units, relative to the B tile
+    if constexpr (DGRAD) {
+#pragma unroll
+        for (int k8 = 0; k8 < KS; ++k8)
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) {
+                const int col = wn0 + tn * MF + li;
+                bq_off[k8][tn] = A_FLOATS / 4 + col * CH + ((LG * k8 + lg) ^ (col % CH));
+            }
+    }
 
     // Read unit u of half h of the stage at float offset st into F.
     auto read_unit = [&](HalfFrag &F, int st, int h, int u) __attribute__((always_inline)) {
-        const int k8l = u / (TM + 2 * TN), v = u % (TM + 2 * TN);
+        const int k8l = u / (TM + NUB), v = u % (TM + NUB);
         const int k8 = h * KH + k8l;
         if (v < TM) {
             F.a[k8l][v] = reinterpret_cast<const float4 *>(smem)[st / 4 + a_off[k8][v]];
+        } else if constexpr (DGRAD) {
+            F.bq[k8l][v - TM] = reinterpret_cast<const float4 *>(smem)[st / 4 + bq_off[k8][v - TM]];
         } else {
             const int tn = (v - TM) / 2, tp = (v - TM) % 2;
             F.b[k8l][2 * tp][tn] = smem[st + b_off + k8 * LG * BROW4 + (2 * tp) * BN + tn * MF];
@@ -680,37 +711,79 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
     //     then this thread's copies of step s+NSTAGE into that slot, one per MFMA, and the LDS
     //     reads of F1 of step s+1.
     //
-    // The fold of a finished position into Y (up to 4*TM*TN vector adds) is dealt out the same
-    // way over the first step of the next position, which accumulates into the other of two
-    // product buffers and starts its chains from a zero accumulator.
+    // What happens to a finished position (the fold into Y, up to 4*TM*TN vector adds, or the stores of
+    // its product tiles) is dealt out the same way over the first step of the next position, which accumulates
+    // into the other of two product buffers and starts its chains from a zero accumulator.
     int st_cur = 0;  // float offset of the ring slot of the current step
     Acc P[2][TM][TN];
     const Acc zero16 = {};
 
-    // Fold unit e of position `pos` (e = j*TM*TN + tm*TN + tn): Y_j +-= P.  The empty asm pins the
+    // Forward.  Fold unit e of position `pos` (e = j*TM*TN + tm*TN + tn): Y_j +-= P.  The empty asm pins the
     // update here: Y is not read again until the final stores, so without it the compiler defers
     // all the adds to the end and keeps the 16 product tiles alive instead of the 4 sums.
-    constexpr int NE = 4 * TM * TN;
-    auto fold_unit = [&](const Acc (&Pp)[TM][TN], int pos, int e) __attribute__((always_inline)) {
-        constexpr unsigned long long plus = kPlus, minus = kMinus;
-        const int j = e / (TM * TN), tm = (e / TN) % TM, tn = e % TN;
-        const int bit = 4 * pos + j;
-        if (ABL & 32) {
-            if (pos == 15) Y[j][tm][tn] += Pp[tm][tn];
-        } else if ((plus >> bit) & 1ull) {
-            Y[j][tm][tn] += Pp[tm][tn];
-            asm volatile("" : "+v"(Y[j][tm][tn]));
-        } else if ((minus >> bit) & 1ull) {
-            Y[j][tm][tn] -= Pp[tm][tn];
-            asm volatile("" : "+v"(Y[j][tm][tn]));
+    // Dgrad.  Unit e = tm*TN + tn: the product tile goes to plane `pos` of Out, written through (the gather
+    // kernel that reads the planes next finds them in the Infinity Cache).  Register r of lane (lg, li) holds
+    // row 4*lg + r, column li of a 16x16 tile; 8*(r/4) + 4*lg + r%4 of a 32x32 tile.
+    constexpr int NE = DGRAD ? TM * TN : 4 * TM * TN;
+    // dgrad: byte offset of this lane's first row and column within the workgroup's rows of a plane; what tile,
+    // register and position add to it is the same for the whole wave, so a store is one instruction with a
+    // scalar base and this offset, and whether a tile lies wholly inside the valid rows and columns is a scalar
+    // test (only a ragged last tile takes per-lane predicates).
+    const unsigned lane_off = (static_cast<unsigned>(wm0 + 4 * lg) * static_cast<unsigned>(N) + n0 + wn0 + li) * 4u;
+    char *const out_tile = reinterpret_cast<char *>(DGRAD ? Out + m0 * N : Out);  // dgrad: this workgroup's first row in plane 0
+    const unsigned rows_u = __builtin_amdgcn_readfirstlane(rows_valid);
+    // dgrad: the product stores count on the same counter as the copies, and memory operations complete in the
+    // order they were issued, so the wait for a tile must allow for the stores issued after its copies.  Their
+    // number is known (REGS per tile) while every tile of the wave lies inside the valid rows and columns (`exact`);
+    // a wave with a ragged tile waits for everything instead.
+    const bool exact = DGRAD && static_cast<unsigned>(wm0 + TM * MF) <= rows_u && n0 + wn0 + TN * MF <= N;
+    bool stores_behind = false;  // the previous step issued a position's product stores
+    auto finish_unit = [&](const Acc (&Pp)[TM][TN], int pos, int e) __attribute__((always_inline)) {
+        if constexpr (DGRAD) {
+            const int tm = e / TN, tn = e % TN;
+            const bool whole = static_cast<unsigned>(wm0 + tm * MF + MF) <= rows_u && n0 + wn0 + tn * MF + MF <= N;  // uniform
+            char *const tile = out_tile + ((static_cast<size_t>(pos) * M + tm * MF) * N + tn * MF) * 4;
+            const size_t row_bytes = static_cast<size_t>(N) * 4;
+            if (whole) {
+#pragma unroll
+                for (int r = 0; r < Cfg::REGS; ++r) {
+                    const int row_u = MF == 32 ? 8 * (r / 4) + (r % 4) : r;  // + tm*MF in tile, + 4*lg + wm0 in lane_off
+                    store_streaming(reinterpret_cast<float *>(tile + row_u * row_bytes + lane_off), Pp[tm][tn][r]);
+                }
+            } else {
+                const bool col_ok = n0 + wn0 + tn * MF + li < N;
+#pragma unroll
+                for (int r = 0; r < Cfg::REGS; ++r) {
+                    const int row_u = MF == 32 ? 8 * (r / 4) + (r % 4) : r;
+                    if (static_cast<unsigned>(wm0 + tm * MF + 4 * lg + row_u) < rows_valid && col_ok)
+                        store_streaming(reinterpret_cast<float *>(tile + row_u * row_bytes + lane_off), Pp[tm][tn][r]);
+                }
+            }
+        } else {
+            constexpr unsigned long long plus = kPlus, minus = kMinus;
+            const int j = e / (TM * TN), tm = (e / TN) % TM, tn = e % TN;
+            const int bit = 4 * pos + j;
+            if ((plus >> bit) & 1ull) {
+                Y[j][tm][tn] += Pp[tm][tn];
+                asm volatile("" : "+v"(Y[j][tm][tn]));
+            } else if ((minus >> bit) & 1ull) {
+                Y[j][tm][tn] -= Pp[tm][tn];
+                asm volatile("" : "+v"(Y[j][tm][tn]));
+            }
         }
     };
+    // Slot (MFMA index 0 .. 2*NM-1 of the first step of the next position) after which unit e goes.
+    auto finish_slot = [](int e) { return e * (2 * NM) / NE; };
+    // dgrad: product stores of a position's first step that go out in its first half (before the wait for the
+    // next tile) and in its second half (behind it).
+    constexpr int NE1 = (NE * NM + 2 * NM - 1) / (2 * NM);  // units e with finish_slot(e) < NM
+    constexpr int ST1 = DGRAD ? NE1 * Cfg::REGS : 0, ST2 = DGRAD ? (NE - NE1) * Cfg::REGS : 0;
 
-    // One step.  first: the chains start from zero and the fold of position fold_pos (held in
-    // Pprev) rides along; otherwise fold_pos is ignored.
-    auto step = [&](Acc (&Pc)[TM][TN], const Acc (&Pprev)[TM][TN], auto first_tag, auto fold_tag) __attribute__((always_inline)) {
+    // One step.  first: the chains start from zero and the finish of position done_pos (held in
+    // Pprev) rides along; otherwise done_pos is ignored.
+    auto step = [&](Acc (&Pc)[TM][TN], const Acc (&Pprev)[TM][TN], auto first_tag, auto done_tag) __attribute__((always_inline)) {
         constexpr bool first = decltype(first_tag)::value;
-        constexpr int fold_pos = decltype(fold_tag)::value;
+        constexpr int done_pos = decltype(done_tag)::value;
         const int st_next = st_cur + STAGE_FLOATS == NSTAGE * STAGE_FLOATS ? 0 : st_cur + STAGE_FLOATS;
         auto mfma_slot = [&](const HalfFrag &F, int i, bool from_zero) __attribute__((always_inline)) {
             if constexpr (BF16) {
@@ -729,26 +802,33 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
                 const int tn = i % TN, tm = (i / TN) % TM, t = (i / (TN * TM)) % 4, k8l = i / (TN * TM * 4);
                 const float4 a4 = F.a[k8l][tm];
                 const float av = t == 0 ? a4.x : t == 1 ? a4.y : t == 2 ? a4.z : a4.w;
+                float bv;
+                if constexpr (DGRAD) {
+                    const float4 b4 = F.bq[k8l][tn];
+                    bv = t == 0 ? b4.x : t == 1 ? b4.y : t == 2 ? b4.z : b4.w;
+                } else {
+                    bv = F.b[k8l][t][tn];
+                }
                 if constexpr (MF == 32)
-                    Pc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, F.b[k8l][t][tn], from_zero ? zero16 : Pc[tm][tn], 0, 0, 0);
+                    Pc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, from_zero ? zero16 : Pc[tm][tn], 0, 0, 0);
                 else
-                    Pc[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, F.b[k8l][t][tn], from_zero ? zero16 : Pc[tm][tn], 0, 0, 0);
+                    Pc[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, from_zero ? zero16 : Pc[tm][tn], 0, 0, 0);
             }
         };
         // Slots (MFMA indices of the second half) after which the copies and LDS reads go; all
         // behind the barrier that follows MFMA 0.
-        auto copy_slot = [](int c) { return NM > 1 ? 1 + (c / GR * GR) * (NM - 1) / LPS : 0; };
-        auto read_slot = [](int u) { return NM > 1 ? 1 + (u / GR * GR) * (NM - 1) / NU : 0; };
+        auto copy_slot = [](int c) { return NM > 1 ? 1 + c * (NM - 1) / LPS : 0; };
+        auto read_slot = [](int u) { return NM > 1 ? 1 + u * (NM - 1) / NU : 0; };
 #pragma unroll
         for (int i = 0; i < NM; ++i) {
             mfma_slot(F1, i, first && i < TM * TN);
 #pragma unroll
             for (int u = 0; u < NU; ++u)
-                if ((u / GR * GR) * NM / NU == i && !(ABL & 8)) read_unit(F2, st_cur, 1, u);
-            if (first && fold_pos >= 0) {
+                if (u * NM / NU == i) read_unit(F2, st_cur, 1, u);
+            if (first && done_pos >= 0) {
 #pragma unroll
                 for (int e = 0; e < NE; ++e)
-                    if ((e / GF * GF) * (2 * NM) / NE == i) fold_unit(Pprev, fold_pos, e);
+                    if (finish_slot(e) == i) finish_unit(Pprev, done_pos, e);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -758,26 +838,39 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
             if (i == 0) {
                 // The tile of the next step is complete once at most the copies of the NSTAGE-2
                 // steps after it are outstanding.
-                if (!(ABL & 2)) wait_vmcnt<(NSTAGE - 2) * LPS>();
+                if constexpr (DGRAD) {
+                    // Newer than the copies of the tile waited for: the copies of the NSTAGE-2 steps after it, the
+                    // stores that went out with the previous step's copies (NSTAGE > 2), and this step's own so far.
+                    constexpr int mine = first && done_pos >= 0 ? ST1 : 0;
+                    if (!exact)
+                        wait_vmcnt<0>();
+                    else if (stores_behind && NSTAGE > 2)
+                        wait_vmcnt<(NSTAGE - 2) * LPS + ST2 + mine>();
+                    else
+                        wait_vmcnt<(NSTAGE - 2) * LPS + mine>();
+                } else {
+                    wait_vmcnt<(NSTAGE - 2) * LPS>();
+                }
                 __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS reads of this step are done
-                if (!(ABL & 1)) __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
             }
 #pragma unroll
             for (int c = 0; c < LPS; ++c)
-                if (copy_slot(c) == i && !(ABL & 4)) copy(c);
+                if (copy_slot(c) == i) copy(c);
 #pragma unroll
             for (int u = 0; u < NU; ++u)
-                if (read_slot(u) == i && !(ABL & 8)) read_unit(F1, st_next, 0, u);
-            if (first && fold_pos >= 0) {
+                if (read_slot(u) == i) read_unit(F1, st_next, 0, u);
+            if (first && done_pos >= 0) {
 #pragma unroll
                 for (int e = 0; e < NE; ++e)
-                    if ((e / GF * GF) * (2 * NM) / NE == NM + i) fold_unit(Pprev, fold_pos, e);
+                    if (finish_slot(e) == NM + i) finish_unit(Pprev, done_pos, e);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
         advance();
         st_cur = st_next;
+        stores_behind = DGRAD && first && done_pos >= 0;
     };
 
     // The position loop is unrolled at compile time so that the signs of the output transform
@@ -789,12 +882,50 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
             step(P[pos & 1], P[(pos & 1) ^ 1], std::false_type{}, std::integral_constant<int, -1>{});
     });
 #pragma unroll
-    for (int e = 0; e < NE; ++e) fold_unit(P[1], 15, e);
+    for (int e = 0; e < NE; ++e) finish_unit(P[1], 15, e);
 
     // The surplus copies must have landed before this workgroup's LDS can be handed on.
     wait_vmcnt<0>();
 
-    if (!(ABL & 16) || nH < 0) store_output<Cfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
+    if constexpr (!DGRAD) store_output<Cfg>(Y, Out, rows_valid, N, nW, m0, n0, wm0, wn0, li, lg, ep);
+}
+
+// Forward: Out [B,2nH,2nW,K] from TI [16][M][C] and Wt [16][C][K].
+// Requirements checked by the launcher: C % BK == 0, K % 4 == 0, TI and Wt 16-byte aligned,
+// tile offsets below 2^31 bytes.  Rows beyond M and columns beyond K are not zero-filled but
+// clamped to the last valid row / column group: what they produce lands in accumulator rows
+// and columns that are never stored.
+template <typename Cfg, int NSTAGE, bool BF16 = false>
+__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_mfma_async_kernel(
+    const float *__restrict__ TI, const float *__restrict__ Wt, float *__restrict__ Out, size_t M, int C, int K, int nH,
+    int nW, unsigned tiles_n, unsigned rows_per_wg, ConvEpilogue ep)
+{
+    const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
+    // The workgroup's tile starts at row m0 and is BM rows tall, of which the first rows_valid are
+    // its own (rows_per_wg <= BM lets the launcher split M evenly at 16-row granularity).
+    const size_t m0 = static_cast<size_t>(lid / tiles_n) * rows_per_wg;
+    const int n0 = static_cast<int>(lid % tiles_n) * Cfg::BN;
+    const unsigned rows_valid = static_cast<unsigned>(M - m0 < rows_per_wg ? M - m0 : rows_per_wg);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same for the whole wave: scalar
+    const int wm0 = (wave / Cfg::WGN) * Cfg::WM, wn0 = (wave % Cfg::WGN) * Cfg::WN;
+    conv_ring_body<Cfg, NSTAGE, BF16, RING_FORWARD>(TI, Wt, Out, M, C, K, nW, m0, n0, rows_valid, wm0, wn0, ep);
+}
+
+// Data gradient: dTI [16][M][C] from dP [16][M][K] and W [16][C][K]: dTI_i = dP_i . W_i^T.
+// Requirements checked by the launcher: K % BK == 0 (the reduction), dP and W 16-byte aligned, tile offsets
+// below 2^31 bytes.  Rows beyond M and columns beyond C are clamped on load and never stored.
+template <typename Cfg, int NSTAGE>
+__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_dgrad_async_kernel(
+    const float *__restrict__ dP, const float *__restrict__ Wt, float *__restrict__ dTI, size_t M, int C, int K,
+    unsigned tiles_n, unsigned rows_per_wg)
+{
+    const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
+    const size_t m0 = static_cast<size_t>(lid / tiles_n) * rows_per_wg;
+    const int n0 = static_cast<int>(lid % tiles_n) * Cfg::BN;
+    const unsigned rows_valid = static_cast<unsigned>(M - m0 < rows_per_wg ? M - m0 : rows_per_wg);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same for the whole wave: scalar
+    const int wm0 = (wave / Cfg::WGN) * Cfg::WM, wn0 = (wave % Cfg::WGN) * Cfg::WN;
+    conv_ring_body<Cfg, NSTAGE, false, RING_DGRAD>(dP, Wt, dTI, M, K, C, 0, m0, n0, rows_valid, wm0, wn0, ConvEpilogue());
 }
 
 }  // namespace

@@ -6,11 +6,12 @@
 // (winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans_grad_cuda.cu.cc:118-129).
 //
 // Conv grad keeps the reference's structure: dP = A dY A^T into the caller's 16*M*K temporary,
-// then two batched GEMMs.  dTI = dP . W^T is a plain library GEMM (rocBLAS strided-batched SGEMM
-// where the reference calls cublasSgemmBatched).  dW = TI^T . dP reduces over the tens of thousands
-// of rows of M into a tiny output, a shape the library handles poorly (31 TFLOP/s at ResNet-18
-// conv3); it runs on the split-reduction MFMA kernel of winograd2x2_wgrad_kernel.h, with rocBLAS
-// kept for the shapes that kernel does not take.  ImTrans grad is one gather kernel: a lane
+// then two batched GEMMs, both on this library's own MFMA kernels (the reference calls cublasSgemmBatched
+// twice).  dTI = dP . W^T walks the 16 positions per workgroup like the forward kernel and stores each
+// product plane as it is finished (conv_dgrad_async_kernel, winograd2x2_conv_kernel.h).  dW = TI^T . dP
+// reduces over the tens of thousands of rows of M into a tiny output; it runs on the split-reduction kernel of
+// winograd2x2_wgrad_kernel.h.  Shapes neither takes (odd channel counts, unaligned pointers) go to one
+// plain tiled kernel.  ImTrans grad is one gather kernel: a lane
 // produces the 2x2 input pixels its tile is centred on from the entries of B dT B^T that fall on
 // them -- its own tile's and the up to 8 neighbouring tiles', handed over through LDS inside a
 // workgroup's block of tiles -- optionally through the fused ReLU's mask; the incoming gradient is
@@ -18,9 +19,8 @@
 
 #include <cstdio>
 
-#include <rocblas/rocblas.h>
-
 #include "swc_common.h"
+#include "winograd2x2_conv_launch.h"
 #include "winograd2x2_wgrad_kernel.h"
 
 namespace swc {
@@ -70,6 +70,7 @@ __global__ __launch_bounds__(256) void output_transform_grad_kernel(const float 
 #pragma unroll
     for (int i = 0; i < 16; ++i) *reinterpret_cast<V *>(dst + i * plane) = p[i];
 }
+
 
 // ---- dX = col2im(B dT B^T) (+ ReLU mask) ----------------------------------------------------------
 // Along one axis, pixel y lies in tile y/2 and in one neighbour; with patch offset r = y + 1 - 2*tile,
@@ -303,15 +304,95 @@ __global__ __launch_bounds__(IG_THREADS) void imtrans_grad_tile_kernel(const flo
         }
 }
 
-// ---- rocBLAS handle: one per host thread and device, created on first use -------------------------
-rocblas_handle blas_handle()
+// ---- any shape, any alignment: Out_i [P x Q] = sum_r A_i(p, r) . B_i(r, q), i = 0..15 ---------------------
+// Element (p, r) of A_i sits at A + i*a_batch + p*a_p + r*a_r (likewise B with b_r, b_q), so the same kernel
+// serves dTI_i = dP_i . W_i^T and dW_i = TI_i^T . dP_i.  A 32x32 output tile per workgroup, 32 reduction
+// indices per step through LDS, one fp32 fma per product: only the shapes the MFMA kernels do not take
+// (C or K not a multiple of 4, M not a multiple of 32, unaligned pointers) come here.
+__global__ __launch_bounds__(256) void gemm16_plain_kernel(const float *__restrict__ A, const float *__restrict__ Bm,
+                                                           float *__restrict__ Out, int P, int Q, int Rn, size_t a_batch,
+                                                           size_t a_p, size_t a_r, size_t b_batch, size_t b_r, size_t b_q,
+                                                           unsigned tiles_q, unsigned tiles_p)
 {
-    constexpr int kMaxDevices = 64;
-    static thread_local rocblas_handle handles[kMaxDevices] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
-    if (handles[dev] == nullptr && rocblas_create_handle(&handles[dev]) != rocblas_status_success) handles[dev] = nullptr;
-    return handles[dev];
+    __shared__ float As[32][33], Bs[32][33];
+    unsigned id = blockIdx.x;
+    const unsigned tq = id % tiles_q;
+    id /= tiles_q;
+    const unsigned tp = id % tiles_p, i = id / tiles_p;
+    const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;  // ty = 0..7
+    const float *a = A + i * a_batch, *b = Bm + i * b_batch;
+    const int p0 = static_cast<int>(tp) * 32, q0 = static_cast<int>(tq) * 32;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int r0 = 0; r0 < Rn; r0 += 32) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int row = ty + 8 * k;  // tile row: p for A, r for B
+            const int pa = p0 + row, ra = r0 + tx;
+            As[row][tx] = pa < P && ra < Rn ? a[pa * a_p + ra * a_r] : 0.f;
+            const int rb = r0 + row, qb = q0 + tx;
+            Bs[row][tx] = rb < Rn && qb < Q ? b[rb * b_r + qb * b_q] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 32; ++r) {
+            const float bv = Bs[r][tx];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) acc[k] = __builtin_fmaf(As[ty + 8 * k][r], bv, acc[k]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int p = p0 + ty + 8 * k, q = q0 + tx;
+        if (p < P && q < Q) Out[(static_cast<size_t>(i) * P + p) * Q + q] = acc[k];
+    }
+}
+
+int gemm16_plain(const float *A, const float *Bm, float *Out, size_t P, int Q, size_t Rn, size_t a_batch, size_t a_p,
+                 size_t a_r, size_t b_batch, size_t b_r, size_t b_q, hipStream_t s)
+{
+    const size_t tiles_p = (P + 31) / 32, tiles_q = (static_cast<size_t>(Q) + 31) / 32;
+    if (16 * tiles_p * tiles_q >= (1ull << 31) || P >= (1ull << 31) || Rn >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
+    gemm16_plain_kernel<<<dim3(static_cast<unsigned>(16 * tiles_p * tiles_q)), dim3(256), 0, s>>>(
+        A, Bm, Out, static_cast<int>(P), Q, static_cast<int>(Rn), a_batch, a_p, a_r, b_batch, b_r, b_q,
+        static_cast<unsigned>(tiles_q), static_cast<unsigned>(tiles_p));
+    return check_launch();
+}
+
+// dTI [16][M][C] = dP [16][M][K] . W [16][C][K]^T on the ring kernel, in the tiling the forward launcher would
+// give a call with these extents (rows M, reduction K, columns C).  SWC_ERR_UNSUPPORTED when no ring tiling
+// takes the shapes.
+template <typename Cfg>
+int launch_dgrad(const float *dP, const float *W, float *dTI, size_t M, int C, int K, size_t rows_per_wg, hipStream_t s)
+{
+    constexpr int kStages = 2;  // a third ring slot (stores waited for a step later) measured 3 % slower
+    constexpr int lds_bytes = async_lds_bytes<Cfg, kStages, RING_DGRAD>();
+    static_assert(lds_bytes <= 160 * 1024, "a CU has 160 KiB of LDS");
+    struct Tag {};
+    const int st = raise_lds_limit<Tag>(reinterpret_cast<const void *>(conv_dgrad_async_kernel<Cfg, kStages>), lds_bytes);
+    if (st != SWC_OK) return st;
+    // Whole MFMA tiles per workgroup, so that only the last row group has a ragged tile (its waves fall back to
+    // waiting for all of their memory operations at every step).
+    rows_per_wg = (rows_per_wg + Cfg::MF - 1) / Cfg::MF * Cfg::MF;
+    const size_t tiles_m = (M + rows_per_wg - 1) / rows_per_wg;
+    const size_t tiles_n = (static_cast<size_t>(C) + Cfg::BN - 1) / Cfg::BN;
+    if (tiles_m * tiles_n >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
+    conv_dgrad_async_kernel<Cfg, kStages><<<dim3(static_cast<unsigned>(tiles_m * tiles_n)), dim3(Cfg::NT), lds_bytes, s>>>(
+        dP, W, dTI, M, C, K, static_cast<unsigned>(tiles_n), static_cast<unsigned>(rows_per_wg));
+    return check_launch();
+}
+
+int dgrad_own(const float *dP, const float *W, float *dTI, size_t M, int C, int K, hipStream_t s)
+{
+    // 32-bit offsets: elements within a workgroup's rows of a plane, bytes within a position's weights
+    if (static_cast<size_t>(112) * C >= (1ull << 30) || static_cast<size_t>(C) * K >= (1ull << 30)) return SWC_ERR_UNSUPPORTED;
+    const TilingChoice pick = choose_tiling(dP, W, M, K, C, false, false);
+    switch (pick.tiling) {
+        case TILING_TALL16: return launch_dgrad<Tall>(dP, W, dTI, M, C, K, pick.rows_per_wg, s);
+        case TILING_SHORT16: return launch_dgrad<Short>(dP, W, dTI, M, C, K, pick.rows_per_wg, s);
+        case TILING_RING32: return launch_dgrad<Tile32>(dP, W, dTI, M, C, K, Tile32::BM, s);
+        default: return SWC_ERR_UNSUPPORTED;
+    }
 }
 
 // dW through the split-reduction kernel.  The partial tiles of the S row splits are parked in the
@@ -350,57 +431,58 @@ int wgrad_own(const float *TI, const float *dP, float *dW, float *scratch, size_
 }  // namespace
 }  // namespace swc
 
-extern "C" int swc_winograd2x2_conv_grad(const float *TInput, const float *Weight, const float *Output_grad,
-                                         float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,
-                                         long long *tmp_ptr_buffer, int C, int B, int H, int W, int K, int pad_h,
-                                         int pad_w, swc_stream_t stream)
+namespace swc {
+namespace {
+
+// The whole backward of the convolution; dP is the 16*M*K-float buffer that holds A dY A^T between the kernels.
+int conv_grad_impl(const float *TInput, const float *Weight, const float *Output_grad, float *TInput_grad,
+                   float *Weight_grad, float *dP, int C, int B, int H, int W, int K, int pad_h, int pad_w, hipStream_t s)
 {
-    using namespace swc;
-    (void)tmp_ptr_buffer;
     if (TInput == nullptr || Weight == nullptr || Output_grad == nullptr || TInput_grad == nullptr ||
-        Weight_grad == nullptr || tmp_data_buffer == nullptr)
+        Weight_grad == nullptr || dP == nullptr)
         return SWC_ERR_NULL_POINTER;
     if (C <= 0 || B <= 0 || H <= 0 || W <= 0 || K <= 0 || (H & 1) || (W & 1)) return SWC_ERR_BAD_DIMS;  // H = 2nH, W = 2nW
     if (pad_h != 1 || pad_w != 1) return SWC_ERR_BAD_PAD;
     const int nH = H / 2, nW = W / 2;
     const size_t M = static_cast<size_t>(B) * nH * nW;
     if (M >= (1ull << 31) || M * K >= (1ull << 32) || M * C >= (1ull << 40)) return SWC_ERR_BAD_DIMS;
-    hipStream_t s = static_cast<hipStream_t>(stream);
 
-    const bool vec = (K % 4 == 0) && aligned16(Output_grad) && aligned16(tmp_data_buffer);
+    const bool vec = (K % 4 == 0) && aligned16(Output_grad) && aligned16(dP);
     const unsigned items = static_cast<unsigned>(M * (vec ? K / 4 : K));
     const dim3 grid((items + 255) / 256), block(256);
     if (vec)
-        output_transform_grad_kernel<4><<<grid, block, 0, s>>>(Output_grad, tmp_data_buffer, nW, K, items, M * K);
+        output_transform_grad_kernel<4><<<grid, block, 0, s>>>(Output_grad, dP, nW, K, items, M * K);
     else
-        output_transform_grad_kernel<1><<<grid, block, 0, s>>>(Output_grad, tmp_data_buffer, nW, K, items, M * K);
+        output_transform_grad_kernel<1><<<grid, block, 0, s>>>(Output_grad, dP, nW, K, items, M * K);
     int st = check_launch();
     if (st != SWC_OK) return st;
 
     // dW first: its partial sums borrow the dTI buffer before the dTI GEMM fills it.
-    st = wgrad_own(TInput, tmp_data_buffer, Weight_grad, TInput_grad, M, C, K, s);
-    const bool dw_done = st == SWC_OK;
-    if (!dw_done && st != SWC_ERR_UNSUPPORTED) return st;
+    st = wgrad_own(TInput, dP, Weight_grad, TInput_grad, M, C, K, s);
+    if (st == SWC_ERR_UNSUPPORTED) {
+        // Row-major dW[i] (C x K) = TI[i]^T (C x M) . dP[i] (M x K): the call at winograd2x2_conv_grad_cuda.cu.cc:115-120.
+        st = gemm16_plain(TInput, dP, Weight_grad, static_cast<size_t>(C), K, M, M * C, 1, static_cast<size_t>(C), M * K,
+                          static_cast<size_t>(K), 1, s);
+    }
+    if (st != SWC_OK) return st;
+    // Row-major dTI[i] (M x C) = dP[i] (M x K) . W[i]^T (K x C): the call at winograd2x2_conv_grad_cuda.cu.cc:103-108.
+    st = dgrad_own(dP, Weight, TInput_grad, M, C, K, s);
+    if (st != SWC_ERR_UNSUPPORTED) return st;
+    return gemm16_plain(dP, Weight, TInput_grad, M, C, static_cast<size_t>(K), M * K, static_cast<size_t>(K), 1,
+                        static_cast<size_t>(C) * K, 1, static_cast<size_t>(K), s);
+}
 
-    rocblas_handle h = blas_handle();
-    if (h == nullptr || rocblas_set_stream(h, s) != rocblas_status_success) return SWC_ERR_HIP;
-    const float one = 1.f, zero = 0.f;
-    const int Mi = static_cast<int>(M);
-    // Row-major dTI[i] (M x C) = dP[i] (M x K) . W[i]^T, as column-major (C x M) = op_T(W: K x C) . (dP: K x M):
-    // the call at winograd2x2_conv_grad_cuda.cu.cc:103-108.
-    rocblas_status rs = rocblas_sgemm_strided_batched(h, rocblas_operation_transpose, rocblas_operation_none, C, Mi, K, &one,
-                                                      Weight, K, static_cast<rocblas_stride>(C) * K, tmp_data_buffer, K,
-                                                      static_cast<rocblas_stride>(M) * K, &zero, TInput_grad, C,
-                                                      static_cast<rocblas_stride>(M) * C, 16);
-    if (rs != rocblas_status_success) return SWC_ERR_HIP;
-    if (dw_done) return SWC_OK;
-    // Row-major dW[i] (C x K) = TI[i]^T . dP[i], as column-major (K x C) = (dP: K x M) . op_T(TI: C x M):
-    // the call at winograd2x2_conv_grad_cuda.cu.cc:115-120.
-    rs = rocblas_sgemm_strided_batched(h, rocblas_operation_none, rocblas_operation_transpose, K, C, Mi, &one,
-                                       tmp_data_buffer, K, static_cast<rocblas_stride>(M) * K, TInput, C,
-                                       static_cast<rocblas_stride>(M) * C, &zero, Weight_grad, K,
-                                       static_cast<rocblas_stride>(C) * K, 16);
-    return rs == rocblas_status_success ? SWC_OK : SWC_ERR_HIP;
+}  // namespace
+}  // namespace swc
+
+extern "C" int swc_winograd2x2_conv_grad(const float *TInput, const float *Weight, const float *Output_grad,
+                                         float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,
+                                         long long *tmp_ptr_buffer, int C, int B, int H, int W, int K, int pad_h,
+                                         int pad_w, swc_stream_t stream)
+{
+    (void)tmp_ptr_buffer;
+    return swc::conv_grad_impl(TInput, Weight, Output_grad, TInput_grad, Weight_grad, tmp_data_buffer, C, B, H, W, K, pad_h,
+                               pad_w, static_cast<hipStream_t>(stream));
 }
 
 namespace swc {

@@ -21,6 +21,7 @@ SWC_ERR_UNSUPPORTED = -6
 # Every symbol include/winograd2x2.h declares with C linkage.
 C_SYMBOLS = (
     "swc_strerror", "swc_last_hip_error", "swc_version", "swc_winograd2x2_conv_last_kernel",
+    "swc_winograd2x2_conv_force_tiling",
     "swc_winograd2x2_imtrans", "swc_winograd2x2_imtrans_affine", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
     "swc_winograd2x2_conv_epilogue",
     "swc_winograd2x2_imtrans_bf16out", "swc_winograd2x2_weights_bf16", "swc_winograd2x2_conv_bf16in",
@@ -74,6 +75,8 @@ def lib():
         L.swc_version.argtypes = []
         L.swc_winograd2x2_conv_last_kernel.restype = ctypes.c_char_p
         L.swc_winograd2x2_conv_last_kernel.argtypes = []
+        L.swc_winograd2x2_conv_force_tiling.restype = i32
+        L.swc_winograd2x2_conv_force_tiling.argtypes = [ctypes.c_char_p]
         L.swc_winograd2x2_imtrans.restype = i32
         L.swc_winograd2x2_imtrans.argtypes = [fp, fp] + [i32] * 7 + [vp]
         L.swc_winograd2x2_imtrans_affine.restype = i32
