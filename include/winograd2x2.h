@@ -5,7 +5,8 @@
  * entry point allocates or frees device memory or synchronises: work is queued on
  * `stream` (a hipStream_t passed as void*; NULL is the null stream) and the call
  * returns.  Calls are re-entrant and thread-safe, and keep no state between calls
- * (the one exception says so: swc_winograd2x2_conv_force_tiling sets a per-thread choice).
+ * (the two exceptions say so: swc_winograd2x2_conv_grad_static shares one fixed
+ * scratch array per GPU, swc_winograd2x2_conv_force_tiling sets a per-thread choice).
  *
  * Citations name the interface of the reference (xingyul/sparse-winograd-cnn) that
  * each entry point stands in for; paths are relative to the reference checkout.
@@ -32,6 +33,7 @@ typedef void *swc_stream_t;
 #define SWC_ERR_HIP (-4)          /* the HIP runtime refused the launch; see swc_last_hip_error() */
 #define SWC_ERR_BAD_RANK (-5)     /* op-level wrappers: wrong tensor rank or leading dimension */
 #define SWC_ERR_UNSUPPORTED (-6)  /* valid arguments that this entry point has no kernel for (see its comment) */
+#define SWC_ERR_TOO_LARGE (-7)    /* valid arguments that need more than this entry point's fixed scratch memory */
 
 SWC_API const char *swc_strerror(int status);
 /* hipError_t of the most recent failed launch on the calling thread (0 if none). */
@@ -253,6 +255,20 @@ SWC_API int swc_winograd2x2_conv_grad(const float *TInput, const float *Weight, 
                                       float *TInput_grad, float *Weight_grad, float *tmp_data_buffer,
                                       long long *tmp_ptr_buffer, int C, int B, int H, int W, int K,
                                       int pad_h, int pad_w, swc_stream_t stream);
+
+/*
+ * swc_winograd2x2_conv_grad for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc); it has no counterpart in the reference.  Same arguments and
+ * results without the two temporaries: the 16*B*nH*nW*K floats of A dY A^T are kept in a fixed array in device
+ * memory that the library holds on every GPU it runs on (SWC_CONV_GRAD_STATIC_MAX_FLOATS floats = 64 MiB, i.e.
+ * B*nH*nW*K <= 1 048 576; larger calls return SWC_ERR_TOO_LARGE and launch nothing).  Nothing is allocated or
+ * freed, by this call or by anything it calls.  All calls on one GPU share that array: calls that may overlap on
+ * one GPU (different streams or host threads) race on it and must be serialised by the caller.
+ */
+#define SWC_CONV_GRAD_STATIC_MAX_FLOATS (16u << 20)
+SWC_API int swc_winograd2x2_conv_grad_static(const float *TInput, const float *Weight, const float *Output_grad,
+                                             float *TInput_grad, float *Weight_grad, int C, int B, int H, int W,
+                                             int K, int pad_h, int pad_w, swc_stream_t stream);
 
 /*
  * Gradient of swc_winograd2x2_imtrans: TransIm_grad [16,B,nH,nW,C] -> Input_grad [B,H,W,C].

@@ -32,6 +32,7 @@ extern "C" const char *swc_strerror(int status)
         case SWC_ERR_HIP: return "the HIP runtime refused the launch (see swc_last_hip_error)";
         case SWC_ERR_BAD_RANK: return "wrong tensor rank or leading dimension";
         case SWC_ERR_UNSUPPORTED: return "this entry point has no kernel for these (valid) arguments";
+        case SWC_ERR_TOO_LARGE: return "the arguments need more than this entry point's fixed scratch memory";
         default: return "unknown status";
     }
 }

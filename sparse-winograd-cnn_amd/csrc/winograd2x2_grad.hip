@@ -18,6 +18,7 @@
 // not modified (the reference transforms it in place first, :124).
 
 #include <cstdio>
+#include <mutex>
 
 #include "swc_common.h"
 #include "winograd2x2_conv_launch.h"
@@ -483,6 +484,58 @@ extern "C" int swc_winograd2x2_conv_grad(const float *TInput, const float *Weigh
     (void)tmp_ptr_buffer;
     return swc::conv_grad_impl(TInput, Weight, Output_grad, TInput_grad, Weight_grad, tmp_data_buffer, C, B, H, W, K, pad_h,
                                pad_w, static_cast<hipStream_t>(stream));
+}
+
+// ---- the same backward pass for callers that cannot allocate ------------------------------------------------------
+// The dP buffer lives in a fixed array in device memory (each GPU the library runs on holds its own copy until the
+// process ends).  In host code the array's name stands for the symbol, not for a device address: the address on the
+// current device comes from hipGetSymbolAddress, once per device, and only that pointer is handed to kernels.
+namespace swc {
+namespace {
+
+constexpr size_t kStaticScratchFloats = SWC_CONV_GRAD_STATIC_MAX_FLOATS;
+__device__ __align__(256) float scratch[kStaticScratchFloats];
+
+float *static_scratch(int *status)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static float *ptrs[kMaxDevices] = {};
+    int dev = 0;
+    const hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        *status = e != hipSuccess ? note_hip_error(e) : SWC_ERR_HIP;
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptrs[dev] == nullptr) {
+        void *p = nullptr;
+        const hipError_t es = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (es != hipSuccess || p == nullptr) {
+            *status = es != hipSuccess ? note_hip_error(es) : SWC_ERR_HIP;
+            return nullptr;
+        }
+        ptrs[dev] = static_cast<float *>(p);
+    }
+    *status = SWC_OK;
+    return ptrs[dev];
+}
+
+}  // namespace
+}  // namespace swc
+
+extern "C" int swc_winograd2x2_conv_grad_static(const float *TInput, const float *Weight, const float *Output_grad,
+                                                float *TInput_grad, float *Weight_grad, int C, int B, int H, int W, int K,
+                                                int pad_h, int pad_w, swc_stream_t stream)
+{
+    if (C <= 0 || B <= 0 || H <= 0 || W <= 0 || K <= 0 || (H & 1) || (W & 1)) return SWC_ERR_BAD_DIMS;
+    const size_t need = static_cast<size_t>(16) * B * (H / 2) * (W / 2) * K;  // floats of dP
+    if (need > swc::kStaticScratchFloats) return SWC_ERR_TOO_LARGE;
+    int st = SWC_OK;
+    float *dP = swc::static_scratch(&st);
+    if (dP == nullptr) return st;
+    return swc::conv_grad_impl(TInput, Weight, Output_grad, TInput_grad, Weight_grad, dP, C, B, H, W, K, pad_h, pad_w,
+                               static_cast<hipStream_t>(stream));
 }
 
 namespace swc {

@@ -17,11 +17,12 @@ SWC_ERR_BAD_PAD = -3
 SWC_ERR_HIP = -4
 SWC_ERR_BAD_RANK = -5
 SWC_ERR_UNSUPPORTED = -6
+SWC_ERR_TOO_LARGE = -7
 
 # Every symbol include/winograd2x2.h declares with C linkage.
 C_SYMBOLS = (
     "swc_strerror", "swc_last_hip_error", "swc_version", "swc_winograd2x2_conv_last_kernel",
-    "swc_winograd2x2_conv_force_tiling",
+    "swc_winograd2x2_conv_force_tiling", "swc_winograd2x2_conv_grad_static",
     "swc_winograd2x2_imtrans", "swc_winograd2x2_imtrans_affine", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
     "swc_winograd2x2_conv_epilogue",
     "swc_winograd2x2_imtrans_bf16out", "swc_winograd2x2_weights_bf16", "swc_winograd2x2_conv_bf16in",
@@ -77,6 +78,8 @@ def lib():
         L.swc_winograd2x2_conv_last_kernel.argtypes = []
         L.swc_winograd2x2_conv_force_tiling.restype = i32
         L.swc_winograd2x2_conv_force_tiling.argtypes = [ctypes.c_char_p]
+        L.swc_winograd2x2_conv_grad_static.restype = i32
+        L.swc_winograd2x2_conv_grad_static.argtypes = [fp] * 5 + [i32] * 7 + [vp]
         L.swc_winograd2x2_imtrans.restype = i32
         L.swc_winograd2x2_imtrans.argtypes = [fp, fp] + [i32] * 7 + [vp]
         L.swc_winograd2x2_imtrans_affine.restype = i32
