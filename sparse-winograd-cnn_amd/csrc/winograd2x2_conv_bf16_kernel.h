@@ -39,9 +39,7 @@ struct HbCfg {
 };
 
 // Requires C % BK == 0 and 16-byte aligned TI16 / Wt16.  M < 2^31.  grid.x = ceil(M / rows_per_wg) * tiles_n.
-// ABL: timing ablations for development (bit 0: no barrier, 1: no copy wait, 2: no copies, 3: no LDS
-// reads, 4: no MFMA, 6: no output stores); results are wrong with any bit set.  Always 0 in the library.
-template <typename Cfg, int ABL = 0>
+template <typename Cfg>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_bf16_stored_kernel(
     const unsigned short *__restrict__ TI16, const unsigned short *__restrict__ Wt16, float *__restrict__ Out, size_t M,
     int C, int K, int nH, int nW, unsigned tiles_n, unsigned rows_per_wg, ConvEpilogue ep)
@@ -136,21 +134,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
         // The tiles of the step to fetch have landed once at most the copies of the NSTAGE-2 steps
         // issued after it are outstanding; after the barrier every wave has also finished reading the
         // slot that the next copies overwrite (it was fetched one step earlier still).
-        if (!(ABL & 2)) wait_vmcnt<(NSTAGE - 2) * Cfg::COPIES>();
+        wait_vmcnt<(NSTAGE - 2) * Cfg::COPIES>();
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's own reads of the slot about to be refilled are done
-        if (!(ABL & 1)) __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (!(ABL & 4)) issue();
+        issue();
 #pragma unroll
         for (int h = 0; h < Cfg::NMFMA; ++h) {
-            if (ABL & 8) {
-                fa[set][h] = bf16x8{};
-                fb[set][h] = bf16x8{};
-                asm volatile("" : "+v"(fa[set][h]), "+v"(fb[set][h]));
-            } else {
-                fa[set][h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_next + a_off[h]);
-                fb[set][h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_next + b_off[h]);
-            }
+            fa[set][h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_next + a_off[h]);
+            fb[set][h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_next + b_off[h]);
         }
         st_next = st_next + Cfg::STAGE_BYTES == Cfg::LDS_BYTES ? 0 : st_next + Cfg::STAGE_BYTES;
     };
@@ -161,12 +153,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
         floatx16 P = {};
         auto mfmas = [&](int set) __attribute__((always_inline)) {
 #pragma unroll
-            for (int h = 0; h < Cfg::NMFMA; ++h) {
-                if (ABL & 16)
-                    P[h] += static_cast<float>(fa[set][h][0]) + static_cast<float>(fb[set][h][0]);
-                else
-                    P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][h], fb[set][h], P, 0, 0, 0);
-            }
+            for (int h = 0; h < Cfg::NMFMA; ++h) P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][h], fb[set][h], P, 0, 0, 0);
         };
         // A position starts with its first step's operands in set 0.  Steps go in pairs so that the set
         // indices are compile-time constants (the sets must stay in registers); an odd last step moves
@@ -204,7 +191,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
     });
     wait_vmcnt<0>();  // the surplus copies must land before the workgroup's LDS is handed on
 
-    if (!(ABL & 64) || nH < 0) store_output<HbStoreCfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
+    store_output<HbStoreCfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
 }
 
 // W [16,C,K] fp32 -> Wt16 [16,K,C] bf16 (round to nearest even).  One lane per output element.

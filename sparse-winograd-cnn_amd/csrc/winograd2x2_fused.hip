@@ -54,9 +54,7 @@ __device__ __forceinline__ float bt_d_b_one(const float (&d)[16])
     return d[5] - d[7] - d[13] + d[15];
 }
 
-// ABL: timing ablations for kernel development (bit 0: no input loads, 1: no transform/LDS writes,
-// 2: no weight copies, 3: no operand reads, 4: no barrier); wrong results with any bit set; 0 in the library.
-template <bool RELU, int ABL = 0>
+template <bool RELU>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void relu_conv_fused_kernel(
     const float *__restrict__ X, const float *__restrict__ Wt, float *__restrict__ Out, size_t M, int H, int W, int C,
     int K, int nH, int nW, unsigned tiles_n)
@@ -177,7 +175,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int it = 0; it < nchunks; ++it) {
         const int cur = it & 1, nxt = cur ^ 1;
         const float *st = smem + cur * FSTAGE_FLOATS;
-        if (it + 1 < nchunks && !(ABL & 1)) load_raw((it + 1) * FBK);
+        if (it + 1 < nchunks) load_raw((it + 1) * FBK);
 
         float4 a[2][2];
         float b[2][2][4];
@@ -193,7 +191,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         static_for<8>([&](auto pp_tag) {
             constexpr int pp = decltype(pp_tag)::value;
             constexpr int buf = pp & 1;
-            if (pp + 1 < 8 && !(ABL & 8)) read_pair(buf ^ 1, 2 * (pp + 1));
+            if (pp + 1 < 8) read_pair(buf ^ 1, 2 * (pp + 1));
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
 #pragma unroll
@@ -203,7 +201,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     P[2 * pp + e] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b[buf][e][t], P[2 * pp + e], 0, 0, 0);
                 }
                 // On the last iteration this rewrites stage `nxt` from stale registers: nobody reads it.
-                if (pp >= 4 && !(ABL & 2)) {
+                if (pp >= 4) {
                     if (t == 0) produce(std::integral_constant<int, (pp >= 4 ? 4 * (pp - 4) : 0) + 0>{}, nxt);
                     if (t == 1) produce(std::integral_constant<int, (pp >= 4 ? 4 * (pp - 4) : 0) + 1>{}, nxt);
                     if (t == 2) produce(std::integral_constant<int, (pp >= 4 ? 4 * (pp - 4) : 0) + 2>{}, nxt);
@@ -217,9 +215,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         // has written its transformed rows; stage `cur` is free once everyone has read it.
         wait_vmcnt<0>();
         __builtin_amdgcn_s_waitcnt(0xc07f);
-        if (!(ABL & 16)) __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (it + 2 < nchunks && !(ABL & 4)) copy_b((it + 2) * FBK, cur);
+        if (it + 2 < nchunks) copy_b((it + 2) * FBK, cur);
     }
 
     // ---- fold the 16 products into the four output tiles, ascending position -------------------

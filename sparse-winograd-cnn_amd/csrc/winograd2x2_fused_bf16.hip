@@ -62,9 +62,7 @@ __device__ __forceinline__ unsigned g_slot(unsigned row, unsigned half) { return
 
 // Requires C % 16 == 0, 16-byte aligned X and Wt16, B*H*W*C < 2^30.  AFFINE: x -> fmaf(x, in_scale[c], in_shift[c])
 // on pixels inside the image before the transform.
-// ABL: timing ablations for development (bit 0: no input loads, 1: no transform/LDS writes, 2: no weight
-// copies, 3: no MFMAs/operand reads, 4: no barrier); wrong results with any bit set; 0 in the library.
-template <bool RELU, bool AFFINE, int ABL = 0>
+template <bool RELU, bool AFFINE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void relu_conv_fused_bf16_kernel(
     const float *__restrict__ X, const float *__restrict__ in_scale, const float *__restrict__ in_shift,
     const unsigned short *__restrict__ Wt16, float *__restrict__ Out, size_t M, int H, int W, int C, int K, int nH,
@@ -136,12 +134,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     auto load_raw = [&](auto set_tag, int c0) __attribute__((always_inline)) {
         constexpr int set = decltype(set_tag)::value;
         const char *xc = reinterpret_cast<const char *>(X + c0);
-        if (ABL & 1) return;
 #pragma unroll
         for (int j = 0; j < 16; ++j) raw[set][j] = *reinterpret_cast<const float4 *>(xc + pix_off[j]);
     };
     auto copy_b = [&](int c0, int stage) __attribute__((always_inline)) {
-        if (ABL & 4) return;
         const unsigned short *wc0 = Wt16 + c0;
         const unsigned dst = smem_base + stage * GSTAGE_BYTES + GA_BYTES + wave * 1024u;
 #pragma unroll
@@ -152,7 +148,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // two channels at a time, which keeps the live temporaries at 32 registers.
     auto produce = [&](auto set_tag, int c0, int stage) __attribute__((always_inline)) {
         constexpr int set = decltype(set_tag)::value;
-        if (ABL & 2) return;
         float sc[4] = {1.f, 1.f, 1.f, 1.f}, sh[4] = {0.f, 0.f, 0.f, 0.f};
         if (AFFINE) {
             const float4 s4 = *reinterpret_cast<const float4 *>(in_scale + c0 + 4 * pq);
@@ -186,7 +181,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     };
     // The 16 MFMAs of a chunk, operands read one position ahead.
     auto consume = [&](int stage) __attribute__((always_inline)) {
-        if (ABL & 8) return;
         const unsigned char *st = gsmem + stage * GSTAGE_BYTES;
         bf16x8 a[2], b[2];
         a[0] = *reinterpret_cast<const bf16x8 *>(st + a_rd_off);
@@ -231,7 +225,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         else
             wait_vmcnt<0>();
         __builtin_amdgcn_s_waitcnt(0xc07f);
-        if (!(ABL & 16)) __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (it + 2 < nchunks) copy_b((it + 2) * GBK, cur);
         if (it + 3 < nchunks) load_raw(std::integral_constant<int, nxt>{}, (it + 3) * GBK);
