@@ -193,13 +193,76 @@ def bench_resnet(args, torch, dev):
     }))
 
 
+# (label, N, H = W, C, K): the layer shapes of ResNet-18-var (imagenet-resnet-transWino-prune.py:117-211) at batch 64
+# and 128, benchmark configs 4a/4b, and a handful of shapes outside the model.
+SWEEP_SHAPES = [(("N%d %dx%d %d->%d" % (n, hw, hw, c, k)), n, hw, c, k)
+                for n in (64, 128)
+                for hw, c, k in ((56, 64, 64), (28, 64, 128), (28, 128, 128), (14, 128, 256), (14, 256, 256), (14, 256, 512),
+                                 (14, 512, 512))] + [
+    ("cfg4b N64 7x7 512->512", 64, 7, 512, 512), ("N32 28x28 128->128", 32, 28, 128, 128), ("N16 56x56 64->64", 16, 56, 64, 64),
+    ("N8 112x112 32->32", 8, 112, 32, 32), ("N48 20x20 192->96", 48, 20, 192, 96), ("N256 14x14 128->128", 256, 14, 128, 128),
+    ("N4 56x56 256->64", 4, 56, 256, 64), ("N100 10x10 320->160", 100, 10, 320, 160),
+    ("N24 28x28 96->192", 24, 28, 96, 192), ("N12 14x14 1024->256", 12, 14, 1024, 256), ("N200 8x8 64->320", 200, 8, 64, 320),
+    ("N2 224x224 32->64", 2, 224, 32, 64), ("N64 12x12 384->384", 64, 12, 384, 384)]
+TILINGS = ("ring32", "ring16", "tall16", "short16")
+
+
+def bench_sweep(args, torch, dev):
+    """For every shape: the fp32 convolution kernel under each tiling it is eligible for (forced through
+    swc_winograd2x2_conv_force_tiling) and under the launcher's own choice.  One JSON line; `rows` holds the table."""
+    import swc_hip
+    L = swc_hip.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    rows, worst = [], 0.0
+    for label, N, hw, C, K in SWEEP_SHAPES:
+        nH = nW = (hw + 1) // 2
+        ti = torch.relu(torch.randn(16, N, nH, nW, C, device=dev))
+        w = torch.randn(16, C, K, device=dev) * 0.05
+        y = torch.empty(N, 2 * nH, 2 * nW, K, device=dev)
+
+        def call():
+            if L.swc_winograd2x2_conv(ti.data_ptr(), w.data_ptr(), y.data_ptr(), None, None, C, N, nH, nW, K, 1, 1, stream) != 0:
+                raise RuntimeError("the conv launcher failed")
+
+        iters = max(args.steps // 4, 20)
+        times = {}
+        for name in TILINGS:
+            if L.swc_winograd2x2_conv_force_tiling(name.encode()) != 0:
+                raise RuntimeError("unknown tiling %s" % name)
+            call()
+            if L.swc_winograd2x2_conv_last_kernel().decode() != name:
+                continue   # not eligible for this shape: the launcher fell back
+            for _ in range(3):
+                call()
+            times[name] = time_loop(call, iters, torch)
+        L.swc_winograd2x2_conv_force_tiling(None)
+        call()
+        pick = L.swc_winograd2x2_conv_last_kernel().decode()
+        for _ in range(3):
+            call()
+        t_pick = time_loop(call, iters, torch)
+        best = min(times, key=times.get)
+        # the launcher's choice measured in the same way as the forced runs (same kernel as times[pick])
+        t_pick = min(t_pick, times.get(pick, t_pick))
+        over = t_pick / times[best] - 1.0
+        worst = max(worst, over)
+        rows.append({"shape": label, "pick": pick, "best": best, "us_pick": round(t_pick * 1e3, 1),
+                     "us": {k: round(v * 1e3, 1) for k, v in times.items()}, "pick_over_best_pct": round(100 * over, 1),
+                     "mfma_frac_pick": round(32.0 * N * nH * nW * C * K / (t_pick * 1e-3) / 1e12 / FP32_MFMA_PEAK_TF, 3)})
+        del ti, w, y
+    print(json.dumps({"metric": "fp32 conv kernel time per tiling, launcher's pick against the best", "unit": "us",
+                      "value": round(100 * worst, 1), "value_is": "worst pick_over_best_pct over the rows",
+                      "n_gpus": 1, "higher_is_better": False, "rows": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg5"],
-                    help="cfg1-cfg4b: one layer; cfg5: the whole ResNet-18-var forward (16 Winograd layers), N=128")
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg5", "sweep"],
+                    help="cfg1-cfg4b: one layer; cfg5: the whole ResNet-18-var forward (16 Winograd layers), N=128; "
+                         "sweep: the fp32 conv kernel under every tiling over the model's layer shapes and a few others")
     ap.add_argument("--batch", type=int, default=128, help="batch size of the cfg5 forward")
     ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16", "bf16_stored"],
                     help="fp32 (the reference's arithmetic); bf16: GEMM operands rounded to bf16 inside the conv "
@@ -251,6 +314,8 @@ def main():
     name = args.workload
     if name == "cfg5":
         return bench_resnet(args, torch, dev)
+    if name == "sweep":
+        return bench_sweep(args, torch, dev)
     B, H, W, C, K, density, kind = WORKLOADS[name]
     nH, nW = (H + 1) // 2, (W + 1) // 2
     M = B * nH * nW

@@ -86,11 +86,12 @@ struct TilingChoice {
 
 // The tiling of a call with M rows, reduction length R and N output columns.  `ring16_ok`: the caller has a
 // 16-index-step variant (the forward fp32 kernel only).
-// Cost = passes x MFMA work of a wave per pass (in 16x16 tiles), weighted by what each kernel
-// measured per unit of that work on MI355X relative to ring32, over the ResNet-18 shapes at
-// batch 64 and 128: tall16 8 % more; short16 10 % more, 15 % more when its 64-index steps are
-// fewer than two per position, but 3 % less while all of its workgroups are resident at once
-// (up to three per CU).
+// Cost = passes x MFMA work of a wave per pass (in 16x16 tiles), weighted by what each kernel measured per
+// unit of that work on MI355X relative to ring32 (`bench.py --workload sweep` times every tiling over the
+// ResNet-18 shapes at batch 64 and 128 and a set of other shapes, and prints the choice made here against the
+// best): tall16 8 % more with one workgroup per CU, 2 % less once a second one is resident (its waits
+// then hide behind the other's MFMAs); short16 10 % more, 3 % less while all of its workgroups are resident at
+// once (up to three per CU), and 2 % on top when a position is a single 64-index step.
 inline TilingChoice choose_tiling(const void *A, const void *B, size_t M, int R, int N, bool forward, bool ring16_ok)
 {
     const size_t cus = device_cus();
@@ -111,9 +112,11 @@ inline TilingChoice choose_tiling(const void *A, const void *B, size_t M, int R,
         return {TILING_SYNC, 64};
     }
     const size_t wgs_short = (M + rows_short - 1) / rows_short * tiles_n;
-    const double w_short = R < 128 ? 1.15 : wgs_short <= 3 * cus ? 0.97 : 1.10;
+    const size_t wgs_tall = (M + rows_tall - 1) / rows_tall * tiles_n;
+    const double w_tall = wgs_tall > cus ? 0.98 : 1.08;
+    const double w_short = (wgs_short <= 3 * cus ? 0.97 : 1.10) * (R < 128 ? 1.02 : 1.0);
     const double cost32 = ok32 ? passes((M + 63) / 64 * tiles_n, cus) * 4.0 : 1e30;
-    const double cost_tall = ok_tall ? passes((M + rows_tall - 1) / rows_tall * tiles_n, cus) * 7.0 * 1.08 : 1e30;
+    const double cost_tall = ok_tall ? passes(wgs_tall, cus) * 7.0 * w_tall : 1e30;
     const double cost_short = ok_short ? passes(wgs_short, cus) * 2.0 * w_short : 1e30;
     if (ok_tall && cost_tall < cost32 && cost_tall <= cost_short) return {TILING_TALL16, rows_tall};
     if (ok_short && cost_short < cost32) return {TILING_SHORT16, rows_short};
