@@ -26,12 +26,38 @@ for _p in (ROOT, PKG):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
-# HBM traffic per launch (bytes), measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
-# what the same counters read for a 128 MiB copy (profiles/*_pmc_traffic.md); None where not measured.
+# Memory traffic per launch (bytes) behind the L2s, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
+# dispatch) and scaled by what the same counters read for a 128 MiB copy: FETCH_SIZE x 2.00, WRITE_SIZE x 1.00
+# (profiles/*_pmc_traffic.md).  Keyed by the kernel variant that was profiled: a run whose launcher picked another
+# one, or a configuration that was not profiled, reports null.
 MEASURED_TRAFFIC = {
-    ("cfg3", "fp32", "conv"): 141.0e6,     # 115.3 MB fetched + 25.69 MB written (algorithmic 129.5 MB)
-    ("cfg3", "fp32", "imtrans"): 131.9e6,  # 29.2 MB fetched + 102.76 MB written (algorithmic 128.45 MB)
+    # (workload, precision, op): (kernel variant, bytes)
+    ("cfg3", "fp32", "conv"): ("tall16", (56346.0 * 2 + 25088.0) * 1024),        # algorithmic 129.5 MB
+    ("cfg3", "fp32", "imtrans"): (None, (12582.0 * 2 + 100455.8) * 1024),         # algorithmic 128.45 MB
+    ("cfg2", "fp32", "conv"): ("tall16", (108090.0 * 2 + 50176.0) * 1024),       # algorithmic 257.2 MB
+    ("cfg2", "fp32", "imtrans"): (None, (25126.2 * 2 + 200811.9) * 1024),
+    ("cfg4a", "fp32", "conv"): ("short16", (45722.0 * 2 + 12544.0) * 1024),      # algorithmic 68.4 MB
+    ("cfg4a", "fp32", "imtrans"): (None, (6310.0 * 2 + 50244.1) * 1024),
+    ("cfg4b", "fp32", "conv"): ("short16", (83452.0 * 2 + 8192.0) * 1024),       # algorithmic 58.7 MB
+    ("cfg4b", "fp32", "imtrans"): (None, (3174.0 * 2 + 32781.9) * 1024),
+    ("cfg3", "bf16_stored", "conv"): ("stored-ring3", (29942.5 * 2 + 25088.0) * 1024),   # algorithmic 77.6 MB
+    ("cfg3", "bf16_stored", "imtrans"): (None, (12584.0 * 2 + 50176.0) * 1024),
+    ("cfg2", "bf16_stored", "conv"): ("stored-ring3", (58817.0 * 2 + 50176.0) * 1024),
+    ("cfg2", "bf16_stored", "imtrans"): (None, (25128.0 * 2 + 100352.0) * 1024),
+    ("cfg4a", "bf16_stored", "conv"): ("stored-ring4", (21878.5 * 2 + 12544.0) * 1024),
+    ("cfg4a", "bf16_stored", "imtrans"): (None, (6312.0 * 2 + 25088.0) * 1024),
+    ("cfg4b", "bf16_stored", "conv"): ("stored-ring4", (45330.2 * 2 + 8192.0) * 1024),
+    ("cfg4b", "bf16_stored", "imtrans"): (None, (3176.0 * 2 + 16384.0) * 1024),
 }
+
+
+def measured_traffic(workload, precision, op, variant=None):
+    """Bytes per launch from the table above if `variant` is the kernel variant that was profiled, else None."""
+    entry = MEASURED_TRAFFIC.get((workload, precision, op))
+    if entry is None or (entry[0] is not None and entry[0] != variant):
+        return None
+    return round(entry[1])
+
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, datasheet
 FP32_MFMA_PEAK_TF = 157.3  # MI355X dense fp32 matrix, datasheet
@@ -274,6 +300,9 @@ def main():
                          "imTrans grad through the fused ReLU) and add a `backward` object to the line")
     ap.add_argument("--no-rotate", dest="rotate", action="store_false",
                     help="skip the extra timing over cycled buffer sets (Infinity Cache defeated)")
+    ap.add_argument("--rotate-only", action="store_true",
+                    help="run only the loops over cycled buffer sets and print their timings: the run to put under "
+                         "rocprofv3 for counters of the cold-buffer case")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="time only eager launches; by default the K steps are also replayed from one captured HIP "
                          "graph and, when that is faster, `value`/`ms_per_step` are the replayed figure "
@@ -380,6 +409,49 @@ def main():
         if call_fused() != 0:
             raise RuntimeError("the fused-layer launcher failed")
 
+    def rotated_timings():
+        """The kernels over buffer sets that are cycled, so that consecutive launches cannot be served from the
+        256 MB Infinity Cache: together the sets are larger than it."""
+        set_bytes = (x.numel() + y.numel()) * 4 + ti.numel() * ti.element_size()
+        n_sets = max(2, -(-3 * 256 * 2 ** 20 // set_bytes))
+        if n_sets * set_bytes >= 64 * 2 ** 30:
+            return None
+        sets = [(x.clone(), torch.empty_like(ti), torch.empty_like(y)) for _ in range(n_sets)]
+        for xs, ts, ys in sets:
+            call_imtrans(xs.data_ptr(), ts.data_ptr(), stream)
+        ptrs = [(a.data_ptr(), b.data_ptr(), c.data_ptr()) for a, b, c in sets]
+        state = {"i": 0}
+
+        def nxt():
+            state["i"] = (state["i"] + 1) % n_sets
+            return ptrs[state["i"]]
+
+        def r_imtrans():
+            a, b, _ = nxt()
+            if call_imtrans(a, b, stream) != 0:
+                raise RuntimeError("the imTrans launcher failed")
+
+        def r_conv():
+            _, b, c = nxt()
+            if call_conv(b, c, stream) != 0:
+                raise RuntimeError("the conv launcher failed")
+
+        def r_step():
+            a, b, c = nxt()
+            if call_imtrans(a, b, stream) != 0 or call_conv(b, c, stream) != 0:
+                raise RuntimeError("step failed")
+
+        for f in (r_imtrans, r_conv, r_step):
+            time_loop(f, n_sets, torch)
+        return {"buffer_sets": n_sets, "MB_per_set": round(set_bytes / 1e6, 1),
+                "ms_imtrans": round(time_loop(r_imtrans, args.steps, torch), 5),
+                "ms_conv": round(time_loop(r_conv, args.steps, torch), 5),
+                "ms_step": round(time_loop(r_step, args.steps, torch), 5)}
+
+    if args.rotate_only:
+        print(json.dumps({"workload": name, "gemm_precision": args.precision, "rotated_buffers": rotated_timings()}))
+        return
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -436,44 +508,7 @@ def main():
     ms_pair = time_loop(step, args.steps, torch)
     ms_fused = time_loop(f_fused, args.steps, torch) if fused_ok else None
 
-    # The same kernels over buffer sets that are cycled, so that consecutive launches cannot be served
-    # from the 256 MB Infinity Cache: together the sets are larger than it.
-    rotated = None
-    set_bytes = (x.numel() + y.numel()) * 4 + ti.numel() * ti.element_size()
-    n_sets = max(2, -(-3 * 256 * 2 ** 20 // set_bytes)) if args.rotate else 0
-    if n_sets and n_sets * set_bytes < 64 * 2 ** 30:
-        sets = [(x.clone(), torch.empty_like(ti), torch.empty_like(y)) for _ in range(n_sets)]
-        for xs, ts, ys in sets:
-            call_imtrans(xs.data_ptr(), ts.data_ptr(), stream)
-        ptrs = [(a.data_ptr(), b.data_ptr(), c.data_ptr()) for a, b, c in sets]
-        state = {"i": 0}
-
-        def nxt():
-            state["i"] = (state["i"] + 1) % n_sets
-            return ptrs[state["i"]]
-
-        def r_imtrans():
-            a, b, _ = nxt()
-            if call_imtrans(a, b, stream) != 0:
-                raise RuntimeError("the imTrans launcher failed")
-
-        def r_conv():
-            _, b, c = nxt()
-            if call_conv(b, c, stream) != 0:
-                raise RuntimeError("the conv launcher failed")
-
-        def r_step():
-            a, b, c = nxt()
-            if call_imtrans(a, b, stream) != 0 or call_conv(b, c, stream) != 0:
-                raise RuntimeError("step failed")
-
-        for f in (r_imtrans, r_conv, r_step):
-            time_loop(f, n_sets, torch)
-        rotated = {"buffer_sets": n_sets, "MB_per_set": round(set_bytes / 1e6, 1),
-                   "ms_imtrans": round(time_loop(r_imtrans, args.steps, torch), 5),
-                   "ms_conv": round(time_loop(r_conv, args.steps, torch), 5),
-                   "ms_step": round(time_loop(r_step, args.steps, torch), 5)}
-        del sets
+    rotated = rotated_timings() if args.rotate else None
     if fused_ok:
         y_fused = y.clone()
         step()  # leave the two-op result in y for the parity gate
@@ -502,7 +537,8 @@ def main():
                          "mfma_TFLOPs": round(tf_conv, 2), "mfma_peak_TFLOPs": BF16_MFMA_PEAK_TF}
     if rotated is not None:
         conv_roofline["frac_rotated"] = round(conv_roofline["frac"] * ms_conv / rotated["ms_conv"], 4)
-    conv_roofline.update({"traffic": MEASURED_TRAFFIC.get((name, args.precision, "conv")),
+    conv_variant = L.swc_winograd2x2_conv_last_kernel().decode()
+    conv_roofline.update({"traffic": measured_traffic(name, args.precision, "conv", conv_variant), "kernel_variant": conv_variant,
                           "algorithmic_flop_per_launch": gemm_flops, "algorithmic_bytes_per_launch": conv_bytes})
 
     ms_best = ms_step if ms_step_graph is None else min(ms_step, ms_step_graph)
@@ -558,7 +594,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs_imtrans / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC.get((name, "fp32", "imtrans")),
+            "traffic": measured_traffic(name, "bf16_stored" if stored else "fp32", "imtrans"),
             "algorithmic_bytes_per_launch": imtrans_bytes,
             # the same kernel over cycled buffer sets: nothing it touches is in the Infinity Cache
             "achieved_rotated": None if rotated is None else round(imtrans_bytes / (rotated["ms_imtrans"] * 1e-3) / 1e9, 1),

@@ -41,10 +41,11 @@ SWC_API int swc_last_hip_error(void);
 /* Library version, "major.minor". */
 SWC_API const char *swc_version(void);
 /* Diagnostic with no counterpart in the reference: the name of the convolution kernel that the calling
- * thread's last swc_winograd2x2_conv / _conv_bf16 call launched ("" before the first): "sync" (any shape
- * and alignment), "ring32" / "ring16" (64x64 tiles, 32- / 16-channel steps), "tall16" / "short16" (row
- * groups of up to 112 / 32 rows, dealt evenly over the CUs).  Which one runs depends only on the shapes
- * and pointer alignment; all give the same results to within the order of the reduction over C. */
+ * thread's last swc_winograd2x2_conv / _conv_bf16 / _conv_epilogue / _conv_bf16in call launched ("" before the
+ * first): "sync" (any shape and alignment), "ring32" / "ring16" (64x64 tiles, 32- / 16-channel steps),
+ * "tall16" / "short16" (row groups of up to 112 / 32 rows, dealt evenly over the CUs); for bf16-stored operands
+ * "stored-ring3" / "stored-ring4" (64x64 tiles, 3- / 4-deep copy ring).  Which one runs depends only on the
+ * shapes and pointer alignment; all give the same results to within the order of the reduction over C. */
 SWC_API const char *swc_winograd2x2_conv_last_kernel(void);
 /* Diagnostic with no counterpart in the reference, for benchmarks and tests that compare the tilings: makes
  * the calling thread's later swc_winograd2x2_conv calls (and the data-gradient GEMM of swc_winograd2x2_conv_grad)

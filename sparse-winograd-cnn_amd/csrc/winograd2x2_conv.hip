@@ -179,7 +179,10 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
     // More resident workgroups hide more of each other's waits once there are enough of them to go round
     // (conv3: 18.7 vs 19.6 us); a grid that leaves CUs with one workgroup does better with the deeper
     // ring (conv4b: 30.8 vs 34.2 us).
-    if (tiles_m * tiles_n > cus)
+    if (tiles_m * tiles_n > cus) {
+        note_conv_kernel("stored-ring3");
         return launch_bf16_stored<Wide>(Input16, Weight16t, Output, M, C, K, nH, nW, rows, tiles_n, ep, s);
+    }
+    note_conv_kernel("stored-ring4");
     return launch_bf16_stored<Deep>(Input16, Weight16t, Output, M, C, K, nH, nW, rows, tiles_n, ep, s);
 }

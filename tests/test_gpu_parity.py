@@ -145,6 +145,28 @@ def test_conv_shapes_reach_every_kernel(dev):
     assert seen == {"sync", "ring32", "ring16", "tall16", "short16"}, seen
 
 
+@pytest.mark.parametrize("tiling", ["ring32", "ring16", "tall16", "short16", "sync"])
+@pytest.mark.parametrize("shape", [(8, 14, 14, 128, 128), (5, 9, 11, 192, 72), (63, 14, 14, 64, 120), (2, 3, 5, 64, 100)])
+def test_conv_fp32_under_every_tiling(oracle, dev, shape, tiling):
+    """The launcher's choice taken away (swc_winograd2x2_conv_force_tiling): every tiling must give the oracle's
+    result on every shape it is eligible for, and the override must report what ran."""
+    import swc_hip
+    L = swc_hip.lib()
+    _, conv = ops()
+    ti, w = conv_inputs(shape, 14, density=0.2)
+    want = oracle.conv(ti, w, acc64=True)
+    assert L.swc_winograd2x2_conv_force_tiling(b"no-such-tiling") == swc_hip.SWC_ERR_UNSUPPORTED
+    assert L.swc_winograd2x2_conv_force_tiling(tiling.encode()) == 0
+    try:
+        got = conv(gpu(ti, dev), gpu(w, dev)).cpu().numpy()
+        assert L.swc_winograd2x2_conv_last_kernel().decode() == tiling   # all four shapes take every tiling
+        assert rel_max(got, want) <= TOL and rel_l1(got, want) <= TOL
+    finally:
+        assert L.swc_winograd2x2_conv_force_tiling(None) == 0
+    conv(gpu(ti, dev), gpu(w, dev))
+    assert L.swc_winograd2x2_conv_last_kernel().decode() in ("ring32", "ring16", "tall16", "short16")
+
+
 @pytest.mark.parametrize("shape", [(3, 3, 3, 32, 32), (2, 4, 4, 5, 7), (2, 3, 5, 36, 100), (8, 9, 9, 128, 72),
                                    (63, 14, 14, 128, 120)])
 def test_conv_fp32_exact_on_integers(oracle, dev, shape):
