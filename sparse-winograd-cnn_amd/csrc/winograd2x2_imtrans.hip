@@ -100,10 +100,28 @@ __device__ __forceinline__ unsigned pack_bf16(float lo, float hi)
     const bf16x2_t p = __builtin_convertvector(floatx2_t{lo, hi}, bf16x2_t);  // v_cvt_pk_bf16_f32, RNE
     return __builtin_bit_cast(unsigned, p);
 }
-__device__ __forceinline__ void store_bf16(unsigned short *p, float v) { through_store(p, static_cast<unsigned short>(pack_bf16(v, 0.f))); }
+typedef unsigned uintx2_t __attribute__((ext_vector_type(2)));
+// OUT: 1 = bf16 planes written through (they stay in the Infinity Cache for the convolution), 2 = bf16 planes
+// streamed past the caches (planes too large to stay there anyway).
+template <int OUT>
+__device__ __forceinline__ void store_bf16(unsigned short *p, float v)
+{
+    const unsigned short h = static_cast<unsigned short>(pack_bf16(v, 0.f));
+    if (OUT == 2)
+        __builtin_nontemporal_store(h, p);
+    else
+        through_store(p, h);
+}
+template <int OUT>
 __device__ __forceinline__ void store_bf16(unsigned short *p, const float4 &v)
 {
-    through_store(p, make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w)));
+    const uint2 h = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
+    if (OUT == 2) {
+        const uintx2_t t = {h.x, h.y};
+        __builtin_nontemporal_store(t, reinterpret_cast<uintx2_t *>(p));
+    } else {
+        through_store(p, h);
+    }
 }
 
 template <int VEC, bool RELU>
@@ -132,7 +150,7 @@ __device__ __forceinline__ void transform_vec(const typename Vec<VEC>::type (&d)
 // AFFINE: every pixel inside the image is first mapped to fma(x, scale[c], shift[c]) (an inference-mode
 // batch normalisation folded into the load); the zero padding stays zero, as it does when the
 // normalisation runs as its own pass before the transform.
-template <int VEC, bool RELU, bool AFFINE, bool BF16OUT, typename Idx>
+template <int VEC, bool RELU, bool AFFINE, int BF16OUT, typename Idx>
 __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__restrict__ X, float *__restrict__ TI,
                                                              const float *__restrict__ scale,
                                                              const float *__restrict__ shift, int H, int W, int C,
@@ -186,7 +204,7 @@ __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__rest
         // the planes are stored as bf16 (round to nearest even): TI is then [16,B,nH,nW,C] of 2-byte elements
         unsigned short *dst16 = reinterpret_cast<unsigned short *>(TI) + static_cast<size_t>(idx) * VEC;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) store_bf16(dst16 + i * plane, t[i]);
+        for (int i = 0; i < 16; ++i) store_bf16<BF16OUT>(dst16 + i * plane, t[i]);
         return;
     }
     float *dst = TI + static_cast<size_t>(idx) * VEC;
@@ -202,11 +220,15 @@ int launch_direct(const float *X, const float *scale, const float *shift, float 
     const size_t items = M * (C / VEC);
     const size_t blocks = (items + 255) / 256;
     const dim3 grid(static_cast<unsigned>(blocks)), block(256);
-    if (bf16_out)
-        imtrans_direct_kernel<VEC, RELU, AFFINE, true, Idx><<<grid, block, 0, stream>>>(
+    // bf16 planes above half the Infinity Cache (128 MiB) cannot stay resident for the convolution: streamed.
+    if (bf16_out && 16 * M * C * 2 > (128ull << 20))
+        imtrans_direct_kernel<VEC, RELU, AFFINE, 2, Idx><<<grid, block, 0, stream>>>(
+            X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
+    else if (bf16_out)
+        imtrans_direct_kernel<VEC, RELU, AFFINE, 1, Idx><<<grid, block, 0, stream>>>(
             X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
     else
-        imtrans_direct_kernel<VEC, RELU, AFFINE, false, Idx><<<grid, block, 0, stream>>>(
+        imtrans_direct_kernel<VEC, RELU, AFFINE, 0, Idx><<<grid, block, 0, stream>>>(
             X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
     return check_launch();
 }
