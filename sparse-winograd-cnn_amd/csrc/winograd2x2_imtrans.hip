@@ -63,20 +63,22 @@ struct Vec<4> {
     static __device__ __forceinline__ float4 zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
 };
 
-// Streaming (nontemporal) stores write the transformed planes around the caches.  Measured at ResNet-18
-// conv3 on buffers that are not already cache-resident, the kernel alone runs at 6.0 TB/s with them and
-// 4.3 TB/s without; but the convolution that consumes the planes next then finds none of them in the
-// 256 MB Infinity Cache, and the pair is 2-3 us slower.  So they are used only when the planes are too
-// large to stay resident anyway (STREAM template flag, chosen by the launcher).
+// How the transformed planes are stored decides where the convolution that reads them next finds them.
+// The planes are written once and read by a later kernel, never by this one.
+//   fp32 planes up to 64 MiB: ordinary stores.  The planes stay in the 256 MB Infinity Cache and the
+//     convolution reads them from there (7x7x512 at batch 64: the pair takes 84 us, 98 us when the planes are
+//     streamed to HBM; 14x14x256: 79 vs 80 us, 52 vs 61 us with the bf16-operand convolution).
+//   fp32 planes above 64 MiB: nontemporal stores, streamed past the caches.  With ordinary stores the kernel
+//     is 45 % slower once its output is not already cache-resident (28x28x128 at batch 64, 103 MB of planes:
+//     31 us against 21 us; every line it writes first evicts a dirty one), and the fp32 convolution, bound by
+//     the matrix pipes, takes the same time either way (pair 86 us warm, 94 us cold with both).  The
+//     bf16-operand convolution over fp32 planes is the one that loses: its pair takes 66 us streamed, 52 us
+//     with ordinary stores.
+//   bf16 planes up to 128 MiB: written through as they are issued (the agent-scope form of a store, sc1) but
+//     still allocated in the Infinity Cache, because the bf16 convolution is bound by reading them (its step
+//     is 25 % slower when they come from HBM); above that they cannot stay resident and are streamed.
+// Two 8-byte agent-scope stores per float4 are not an option for fp32: 43 us instead of 21 us.
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
-// The planes are written once and read by a later kernel, never by this one, so no store is left as a dirty
-// line in the L2s for the write-back that ends the kernel to drain.
-// fp32 planes: nontemporal stores, streamed past the caches.  With ordinary stores the kernel is 40 % slower
-// once its output no longer fits the Infinity Cache (every line it writes first evicts a dirty one); the fp32
-// convolution that reads the planes next is bound by the matrix pipes and runs equally fast either way.
-// bf16 planes: written through as they are issued (the agent-scope form of a store, sc1) but still allocated
-// in the Infinity Cache, because the bf16 convolution is bound by reading them (its step is 25 % slower when
-// they come from HBM).
 __device__ __forceinline__ void stream_store(float *p, float v) { __builtin_nontemporal_store(v, p); }
 __device__ __forceinline__ void stream_store(float *p, const float4 &v)
 {
@@ -101,8 +103,8 @@ __device__ __forceinline__ unsigned pack_bf16(float lo, float hi)
     return __builtin_bit_cast(unsigned, p);
 }
 typedef unsigned uintx2_t __attribute__((ext_vector_type(2)));
-// OUT: 1 = bf16 planes written through (they stay in the Infinity Cache for the convolution), 2 = bf16 planes
-// streamed past the caches (planes too large to stay there anyway).
+// OUT (the kernel's store mode): 0 = fp32 planes streamed, 3 = fp32 planes with ordinary stores,
+// 1 = bf16 planes written through, 2 = bf16 planes streamed.
 template <int OUT>
 __device__ __forceinline__ void store_bf16(unsigned short *p, float v)
 {
@@ -150,7 +152,7 @@ __device__ __forceinline__ void transform_vec(const typename Vec<VEC>::type (&d)
 // AFFINE: every pixel inside the image is first mapped to fma(x, scale[c], shift[c]) (an inference-mode
 // batch normalisation folded into the load); the zero padding stays zero, as it does when the
 // normalisation runs as its own pass before the transform.
-template <int VEC, bool RELU, bool AFFINE, int BF16OUT, typename Idx>
+template <int VEC, bool RELU, bool AFFINE, int OUT, typename Idx>
 __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__restrict__ X, float *__restrict__ TI,
                                                              const float *__restrict__ scale,
                                                              const float *__restrict__ shift, int H, int W, int C,
@@ -200,14 +202,20 @@ __global__ __launch_bounds__(256) void imtrans_direct_kernel(const float *__rest
     }
     V t[16];
     transform_vec<VEC, RELU>(d, t);
-    if (BF16OUT) {
+    if (OUT == 1 || OUT == 2) {
         // the planes are stored as bf16 (round to nearest even): TI is then [16,B,nH,nW,C] of 2-byte elements
         unsigned short *dst16 = reinterpret_cast<unsigned short *>(TI) + static_cast<size_t>(idx) * VEC;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) store_bf16<BF16OUT>(dst16 + i * plane, t[i]);
+        for (int i = 0; i < 16; ++i) store_bf16<OUT>(dst16 + i * plane, t[i]);
         return;
     }
     float *dst = TI + static_cast<size_t>(idx) * VEC;
+    if (OUT == 3) {
+        V *dv = reinterpret_cast<V *>(dst);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dv[i * (plane / VEC)] = t[i];
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 16; ++i) stream_store(dst + i * plane, t[i]);
 }
@@ -220,12 +228,15 @@ int launch_direct(const float *X, const float *scale, const float *shift, float 
     const size_t items = M * (C / VEC);
     const size_t blocks = (items + 255) / 256;
     const dim3 grid(static_cast<unsigned>(blocks)), block(256);
-    // bf16 planes above half the Infinity Cache (128 MiB) cannot stay resident for the convolution: streamed.
+    // Store mode by the size of the planes (see the store helpers above).
     if (bf16_out && 16 * M * C * 2 > (128ull << 20))
         imtrans_direct_kernel<VEC, RELU, AFFINE, 2, Idx><<<grid, block, 0, stream>>>(
             X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
     else if (bf16_out)
         imtrans_direct_kernel<VEC, RELU, AFFINE, 1, Idx><<<grid, block, 0, stream>>>(
+            X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
+    else if (16 * M * C * 4 <= (64ull << 20))
+        imtrans_direct_kernel<VEC, RELU, AFFINE, 3, Idx><<<grid, block, 0, stream>>>(
             X, TI, scale, shift, H, W, C, nH, nW, static_cast<Idx>(items), M * C);
     else
         imtrans_direct_kernel<VEC, RELU, AFFINE, 0, Idx><<<grid, block, 0, stream>>>(
