@@ -36,10 +36,10 @@ MEASURED_TRAFFIC = {
     ("cfg3", "fp32", "imtrans"): (None, (12582.0 * 2 + 100455.8) * 1024),         # algorithmic 128.45 MB
     ("cfg2", "fp32", "conv"): ("tall16", (108090.0 * 2 + 50176.0) * 1024),       # algorithmic 257.2 MB
     ("cfg2", "fp32", "imtrans"): (None, (25126.2 * 2 + 200811.9) * 1024),
-    ("cfg4a", "fp32", "conv"): ("short16", (45722.0 * 2 + 12544.0) * 1024),      # algorithmic 68.4 MB
-    ("cfg4a", "fp32", "imtrans"): (None, (6310.0 * 2 + 50244.1) * 1024),
+    ("cfg4a", "fp32", "conv"): ("short16", (48243.9 * 2 + 12544.0) * 1024),      # algorithmic 68.4 MB
+    ("cfg4a", "fp32", "imtrans"): (None, (6432.0 * 2 + 50176.0) * 1024),
     ("cfg4b", "fp32", "conv"): ("short16", (83452.0 * 2 + 8192.0) * 1024),       # algorithmic 58.7 MB
-    ("cfg4b", "fp32", "imtrans"): (None, (3174.0 * 2 + 32781.9) * 1024),
+    ("cfg4b", "fp32", "imtrans"): (None, (3175.0 * 2 + 32768.0) * 1024),
     ("cfg3", "bf16_stored", "conv"): ("stored-ring3", (29942.5 * 2 + 25088.0) * 1024),   # algorithmic 77.6 MB
     ("cfg3", "bf16_stored", "imtrans"): (None, (12584.0 * 2 + 50176.0) * 1024),
     ("cfg2", "bf16_stored", "conv"): ("stored-ring3", (58817.0 * 2 + 50176.0) * 1024),
