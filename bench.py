@@ -372,7 +372,7 @@ def main():
             return L.swc_winograd2x2_imtrans_bf16out(a, None, None, b, C, B, H, W, 1, 1, 1, st)
 
         def call_conv(b, c, st):
-            return L.swc_winograd2x2_conv_bf16in(b, w16p, c, None, None, None, C, B, nH, nW, K, 1, 1, st)
+            return L.swc_winograd2x2_conv_bf16in(b, w16p, c, None, None, None, 0, C, B, nH, nW, K, 1, 1, st)
     else:
         conv_entry = L.swc_winograd2x2_conv if args.precision == "fp32" else L.swc_winograd2x2_conv_bf16
         winograd2x2_imTrans(x, relu=True, out=ti)

@@ -113,7 +113,9 @@ SWC_API int swc_winograd2x2_conv(const float *Input, const float *Weight, float 
 
 /*
  * swc_winograd2x2_conv with per-element work folded into its output stores:
- *   Output = fmaf(conv, Scale[k], Shift[k]) + Residual
+ *   Output = fmaf(conv, Scale[k], Shift[k]) + Residual        (residual_relu == 0)
+ *   Output = fmaf(conv, Scale[k], Shift[k]) + max(Residual, 0) (residual_relu != 0: the identity shortcut of the
+ *            units without a 1x1 conv is `relu(x)`, imagenet-resnet-transWino-prune.py:135-143)
  *   Scale, Shift [K] fp32 (both or neither); Residual [B,2nH,2nW,K] fp32; any of them may be NULL.
  *   precision: 0 = fp32 MFMA, 1 = bf16 operands (as swc_winograd2x2_conv_bf16).
  * No counterpart function in the reference: it is what follows its second convolution of every
@@ -123,7 +125,7 @@ SWC_API int swc_winograd2x2_conv(const float *Input, const float *Weight, float 
  * Residual may alias Output (each element is read before it is written, by the same lane).
  */
 SWC_API int swc_winograd2x2_conv_epilogue(const float *Input, const float *Weight, float *Output,
-                                  const float *Scale, const float *Shift, const float *Residual,
+                                  const float *Scale, const float *Shift, const float *Residual, int residual_relu,
                                   int C, int B, int nH, int nW, int K, int pad_h, int pad_w,
                                   int precision, swc_stream_t stream);
 
@@ -216,11 +218,11 @@ SWC_API int swc_winograd2x2_imtrans_bf16out(const float *Input, const float *Sca
 SWC_API int swc_winograd2x2_weights_bf16(const float *Weight, uint16_t *Weight16t, int C, int K, swc_stream_t stream);
 
 /* swc_winograd2x2_conv_epilogue over the bf16 operands: Output [B,2nH,2nW,K] fp32 =
- * fmaf(conv, Scale[k], Shift[k]) + Residual (Scale/Shift/Residual may be NULL).  Needs C % 64 == 0 and
+ * fmaf(conv, Scale[k], Shift[k]) + Residual (Scale/Shift/Residual may be NULL; residual_relu as above).  Needs C % 64 == 0 and
  * 16-byte aligned operands; returns SWC_ERR_UNSUPPORTED otherwise (use the fp32-stored path). */
 SWC_API int swc_winograd2x2_conv_bf16in(const uint16_t *Input16, const uint16_t *Weight16t, float *Output,
-                                const float *Scale, const float *Shift, const float *Residual, int C, int B,
-                                int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream);
+                                const float *Scale, const float *Shift, const float *Residual, int residual_relu,
+                                int C, int B, int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream);
 
 /* The whole layer in one kernel with bf16 GEMM operands: the values of swc_winograd2x2_imtrans_bf16out
  * (with InScale/InShift as in swc_winograd2x2_imtrans_affine, or NULL) followed by

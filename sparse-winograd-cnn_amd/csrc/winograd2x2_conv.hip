@@ -108,13 +108,15 @@ extern "C" int swc_winograd2x2_conv_bf16(const float *Input, const float *Weight
 }
 
 extern "C" int swc_winograd2x2_conv_epilogue(const float *Input, const float *Weight, float *Output, const float *Scale,
-                                             const float *Shift, const float *Residual, int C, int B, int nH, int nW,
-                                             int K, int pad_h, int pad_w, int precision, swc_stream_t stream)
+                                             const float *Shift, const float *Residual, int residual_relu, int C, int B,
+                                             int nH, int nW, int K, int pad_h, int pad_w, int precision,
+                                             swc_stream_t stream)
 {
     swc::ConvEpilogue ep;
     ep.scale = Scale;
     ep.shift = Shift;
     ep.residual = Residual;
+    ep.residual_relu = residual_relu != 0;
     if (precision == 0) return swc::conv_entry<false>(Input, Weight, Output, C, B, nH, nW, K, pad_h, pad_w, ep, stream);
     if (precision == 1) return swc::conv_entry<true>(Input, Weight, Output, C, B, nH, nW, K, pad_h, pad_w, ep, stream);
     return SWC_ERR_BAD_DIMS;
@@ -150,8 +152,9 @@ int launch_bf16_stored(const unsigned short *Input16, const unsigned short *Weig
 }  // namespace swc
 
 extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const unsigned short *Weight16t, float *Output,
-                                           const float *Scale, const float *Shift, const float *Residual, int C, int B,
-                                           int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream)
+                                           const float *Scale, const float *Shift, const float *Residual,
+                                           int residual_relu, int C, int B, int nH, int nW, int K, int pad_h, int pad_w,
+                                           swc_stream_t stream)
 {
     using namespace swc;
     if (Input16 == nullptr || Weight16t == nullptr || Output == nullptr) return SWC_ERR_NULL_POINTER;
@@ -175,6 +178,7 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
     ep.scale = Scale;
     ep.shift = Shift;
     ep.residual = Residual;
+    ep.residual_relu = residual_relu != 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // More resident workgroups hide more of each other's waits once there are enough of them to go round
     // (conv3: 18.7 vs 19.6 us); a grid that leaves CUs with one workgroup does better with the deeper

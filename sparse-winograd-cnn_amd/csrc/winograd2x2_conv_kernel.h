@@ -95,12 +95,15 @@ struct ConvCfg {
 template <typename Cfg>
 using AccT = typename std::conditional<Cfg::MF == 32, floatx16, floatx4>::type;
 
-// Optional per-element work folded into the output stores: out = fmaf(y, scale[k], shift[k]) + residual.
+// Optional per-element work folded into the output stores: out = fmaf(y, scale[k], shift[k]) + residual,
+// or + max(residual, 0) with residual_relu (the `relu` that an identity shortcut applies to the unit's input,
+// ResNet-18-var/imagenet-resnet-transWino-prune.py:135-143, without a pass of its own).
 // scale and shift go together; either part may be absent (null).  All null: plain stores.
 struct ConvEpilogue {
     const float *scale = nullptr;     // [K]
     const float *shift = nullptr;     // [K]
     const float *residual = nullptr;  // [B,2nH,2nW,K], the output's layout
+    int residual_relu = 0;
 };
 
 // Output values are written once and not read again by the kernel that writes them.  A plain store leaves
@@ -196,6 +199,12 @@ __device__ __forceinline__ void store_output(const AccT<Cfg> (&Y)[4][Cfg::TM][Cf
         q[2][tm][r][tn] = src[row_stride];
         q[3][tm][r][tn] = src[row_stride + K];
     });
+    if (ep.residual_relu) {  // uniform over the grid
+        for_each_value([&](int tm, int r, int tn, size_t) __attribute__((always_inline)) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) q[j][tm][r][tn] = q[j][tm][r][tn] > 0.f ? q[j][tm][r][tn] : 0.f;
+        });
+    }
     for_each_value([&](int tm, int r, int tn, size_t at) __attribute__((always_inline)) {
         finish(tm, r, tn, at, q[0][tm][r][tn], q[1][tm][r][tn], q[2][tm][r][tn], q[3][tm][r][tn]);
     });

@@ -82,6 +82,21 @@ def _conv_bn_folded(conv, bn):
     return cached[1], cached[2]
 
 
+def _shortcut_folded(conv, bn, bn_out):
+    """The 1x1 shortcut conv + its BatchNorm, for a branch whose last convolution applies ``bn_out`` and adds
+    the shortcut in its stores: returns (Wt [Cin,Cout], scale, shift) such that
+    ``branch*scale + shift + x_nhwc @ Wt == bn_out(branch) + bn(conv(x))``.  A 1x1 convolution over NHWC data is
+    one matrix product, and its bias joins the shift the kernel adds anyway.  Cached like _conv_bn_folded."""
+    w1, b1 = _conv_bn_folded(conv, bn)
+    scale, shift = _bn_affine(bn_out)
+    key = (conv._swc_folded[0], bn_out._swc_affine[0])
+    cached = getattr(conv, "_swc_shortcut", None)
+    if cached is None or cached[0] != key:
+        cached = (key, w1.view(w1.shape[0], w1.shape[1]).t().contiguous(), scale, (shift + b1).contiguous())
+        conv._swc_shortcut = cached
+    return cached[1], cached[2], cached[3]
+
+
 def _to_nhwc(x):   # NCHW tensor in channels_last memory -> contiguous [B,H,W,C] view
     return x.permute(0, 2, 3, 1).contiguous()
 
@@ -109,31 +124,38 @@ class WinogradUnit(torch.nn.Module):
             self.conv1 = torch.nn.Conv2d(c_in, c_out, 1, bias=False)
             self.bn1 = torch.nn.BatchNorm2d(c_out)
 
-    def branch(self, x, shortcut=None):
+    def branch(self, x, shortcut=None, out_affine=None, shortcut_relu=False):
         """The two Winograd layers.  With ``fold_bn`` the three BatchNorms and the residual add run inside
         the Winograd kernels (bn2a, bn2b in the transforms' loads; bn2c and ``+ shortcut`` in the second
-        convolution's stores) and the result is already ``shortcut + branch``."""
+        convolution's stores) and the result is already ``shortcut + branch``; ``shortcut`` is then NHWC and
+        ``out_affine`` replaces bn2c's (scale, shift); ``shortcut_relu``: the kernel adds ``relu(shortcut)``."""
         if self.fold_bn:
             dt = self.ti_dtype
             h = self.conv2a(WinogradImTrans(_to_nhwc(x), torch.relu, affine=_bn_affine(self.bn2a), out_dtype=dt))
             h = self.conv2b(WinogradImTrans(h, torch.relu, affine=_bn_affine(self.bn2b), out_dtype=dt),
-                            affine=_bn_affine(self.bn2c), residual=_to_nhwc(shortcut))
+                            affine=out_affine if out_affine is not None else _bn_affine(self.bn2c), residual=shortcut,
+                            residual_relu=shortcut_relu)
             return _to_nchw(h)
         h = _to_nchw(self.conv2a(WinogradImTrans(_to_nhwc(self.bn2a(x)), torch.relu)))
         h = _to_nchw(self.conv2b(WinogradImTrans(_to_nhwc(self.bn2b(h)), torch.relu)))
         return shortcut + self.bn2c(h)
 
     def forward(self, x):
+        out_affine = None
         if self.shortcut:
             s = torch.relu(self.bn_pre(x)) if self.bn_pre is not None else torch.relu(x)
             if self.fold_bn:
-                w1, b1 = _conv_bn_folded(self.conv1, self.bn1)
-                sc = F.conv2d(s, w1, b1)
+                wt, scale, shift = _shortcut_folded(self.conv1, self.bn1, self.bn2c)
+                s = _to_nhwc(s)
+                sc = torch.mm(s.view(-1, s.shape[3]), wt).view(s.shape[0], s.shape[1], s.shape[2], wt.shape[1])
+                out_affine = (scale, shift)
             else:
                 sc = self.bn1(self.conv1(s))
+        elif self.fold_bn:
+            sc = _to_nhwc(x)   # the identity shortcut relu(x): its ReLU is applied where the kernel reads it
         else:
             sc = torch.relu(x)
-        x = self.branch(x, sc)
+        x = self.branch(x, sc, out_affine, shortcut_relu=self.fold_bn and not self.shortcut)
         if self.pool:
             x = _max_pool_same(x)
         return x

@@ -88,13 +88,13 @@ def lib():
             f.restype = i32
             f.argtypes = [fp, fp, fp, fp, vp] + [i32] * 7 + [vp]
         L.swc_winograd2x2_conv_epilogue.restype = i32
-        L.swc_winograd2x2_conv_epilogue.argtypes = [fp] * 6 + [i32] * 8 + [vp]
+        L.swc_winograd2x2_conv_epilogue.argtypes = [fp] * 6 + [i32] * 9 + [vp]
         L.swc_winograd2x2_imtrans_bf16out.restype = i32
         L.swc_winograd2x2_imtrans_bf16out.argtypes = [fp, fp, fp, fp] + [i32] * 7 + [vp]
         L.swc_winograd2x2_weights_bf16.restype = i32
         L.swc_winograd2x2_weights_bf16.argtypes = [fp, fp, i32, i32, vp]
         L.swc_winograd2x2_conv_bf16in.restype = i32
-        L.swc_winograd2x2_conv_bf16in.argtypes = [fp] * 6 + [i32] * 7 + [vp]
+        L.swc_winograd2x2_conv_bf16in.argtypes = [fp] * 6 + [i32] * 8 + [vp]
         L.swc_winograd2x2_relu_conv_bf16.restype = i32
         L.swc_winograd2x2_relu_conv_bf16.argtypes = [fp] * 8 + [i32] * 8 + [vp]
         L.swc_winograd2x2_imtrans_op_shape.restype = i32

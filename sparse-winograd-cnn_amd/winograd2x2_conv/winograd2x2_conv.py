@@ -42,7 +42,7 @@ def _plan(i_shape, w_shape):
     return plan
 
 
-def _forward(I, W, precision, out, scale=None, shift=None, residual=None):
+def _forward(I, W, precision, out, scale=None, shift=None, residual=None, residual_relu=False):
     if precision not in PRECISIONS:
         raise ValueError("precision must be one of %s" % sorted(PRECISIONS))
     I = swc_hip.require_cuda_f32(I, "I", 5)
@@ -73,7 +73,7 @@ def _forward(I, W, precision, out, scale=None, shift=None, residual=None):
             st = swc_hip.lib().swc_winograd2x2_conv_epilogue(
                 I.data_ptr(), W.data_ptr(), out.data_ptr(), None if scale is None else scale.data_ptr(),
                 None if shift is None else shift.data_ptr(), None if residual is None else residual.data_ptr(),
-                C, B, nH, nW, shape[3], 1, 1, PRECISIONS[precision], stream)
+                int(bool(residual_relu)), C, B, nH, nW, shape[3], 1, 1, PRECISIONS[precision], stream)
         else:
             st = swc_hip.lib().swc_winograd2x2_conv_op_compute(
                 I.data_ptr(), 5, i_dims, W.data_ptr(), 3, w_dims, out.data_ptr(), 4, o_dims, PRECISIONS[precision],
@@ -95,7 +95,7 @@ def winograd2x2_weights_bf16(W):
     return out
 
 
-def _forward_bf16_stored(I, W, out, scale, shift, residual):
+def _forward_bf16_stored(I, W, out, scale, shift, residual, residual_relu=False):
     """I [16,B,nH,nW,C] bfloat16; W [16,C,K] float32 or prepared [16,K,C] bfloat16."""
     I = swc_hip.require_cuda_f32(I, "I", 5, torch.bfloat16)
     if not isinstance(W, torch.Tensor) or W.dim() != 3:
@@ -127,7 +127,7 @@ def _forward_bf16_stored(I, W, out, scale, shift, residual):
         st = swc_hip.lib().swc_winograd2x2_conv_bf16in(
             I.data_ptr(), W.data_ptr(), out.data_ptr(), None if scale is None else scale.data_ptr(),
             None if shift is None else shift.data_ptr(), None if residual is None else residual.data_ptr(),
-            C, B, nH, nW, K, 1, 1, stream)
+            int(bool(residual_relu)), C, B, nH, nW, K, 1, 1, stream)
     swc_hip.check(st, "winograd2x2_conv (bf16-stored operands)")
     return out
 
@@ -169,7 +169,7 @@ class _ConvFunction(torch.autograd.Function):
         return dI, dW, None
 
 
-def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, residual=None):
+def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, residual=None, residual_relu=False):
     """I: [16,B,nH,nW,C], W: [16,C,K], float32 on the GPU -> [B,2nH,2nW,K] (uncropped).
 
     A bfloat16 ``I`` (from ``winograd2x2_imTrans(..., out_dtype=torch.bfloat16)``) takes the bf16-stored
@@ -177,7 +177,8 @@ def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, r
     tensor ``winograd2x2_weights_bf16`` prepared from it.
     ``scale``/``shift`` ([K]) and ``residual`` ([B,2nH,2nW,K]), forward only: the result becomes
     ``conv*scale + shift + residual`` inside the kernel's stores (an inference BatchNorm and the
-    residual add that follow the second convolution of a ResNet unit).
+    residual add that follow the second convolution of a ResNet unit); with ``residual_relu=True`` it is
+    ``... + relu(residual)`` (the identity shortcut of the reference model is ``relu(x)``).
 
     ``precision="bf16"`` rounds both GEMM operands to bf16 (fp32 accumulate).  Differentiable
     through ``winograd2x2_conv_grad`` when an input requires grad.
@@ -186,14 +187,16 @@ def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, r
     if isinstance(I, torch.Tensor) and I.dtype == torch.bfloat16:
         if needs_grad:
             raise NotImplementedError("the bf16-stored variant is forward only")
-        return _forward_bf16_stored(I, W, out, scale, shift, residual)
+        return _forward_bf16_stored(I, W, out, scale, shift, residual, residual_relu)
+    if residual_relu and residual is None:
+        raise ValueError("residual_relu needs a residual")
     if (scale is not None or residual is not None) and needs_grad:
         raise NotImplementedError("the scale/shift/residual epilogue is forward only")
     if needs_grad:
         if out is not None:
             raise NotImplementedError("out= is forward only: the result written there would carry no gradient")
         return _ConvFunction.apply(I, W, precision)
-    return _forward(I, W, precision, out, scale, shift, residual)
+    return _forward(I, W, precision, out, scale, shift, residual, residual_relu)
 
 
 def winograd2x2_relu_conv(X, W, relu=True, out=None):

@@ -80,9 +80,9 @@ class WinogradConv(torch.nn.Module):
             self._masked = cached
         return cached[1]
 
-    def forward(self, x, affine=None, residual=None):
+    def forward(self, x, affine=None, residual=None, residual_relu=False):
         """``affine=(scale, shift)`` and ``residual`` (forward only) are applied to the result inside
-        the kernel: ``conv*scale + shift + residual``."""
+        the kernel: ``conv*scale + shift + residual`` (``+ relu(residual)`` with ``residual_relu``)."""
         if x.dtype == torch.bfloat16:      # bf16-stored activations: forward only
             w = self.bf16_weight()
         elif torch.is_grad_enabled() and self.W.requires_grad:
@@ -91,4 +91,5 @@ class WinogradConv(torch.nn.Module):
             w = self.masked_weight()
         scale, shift = affine if affine is not None else (None, None)
         return winograd2x2_conv.winograd2x2_conv.winograd2x2_conv(x, w, precision=self.precision, scale=scale,
-                                                                  shift=shift, residual=residual)
+                                                                  shift=shift, residual=residual,
+                                                                  residual_relu=residual_relu)

@@ -80,6 +80,9 @@ def test_conv_over_bf16_operands(oracle, dev, shape):
     got2 = winograd2x2_conv(ti_gpu, winograd2x2_weights_bf16(gpu(w, dev)), scale=gpu(scale, dev), shift=gpu(shift, dev),
                             residual=gpu(res, dev)).cpu().numpy()
     assert np.array_equal(got2, oracle.affine(got, scale, shift) + res)
+    got3 = winograd2x2_conv(ti_gpu, winograd2x2_weights_bf16(gpu(w, dev)), scale=gpu(scale, dev), shift=gpu(shift, dev),
+                            residual=gpu(res, dev), residual_relu=True).cpu().numpy()
+    assert np.array_equal(got3, oracle.affine(got, scale, shift) + np.maximum(res, 0))
     # the same values as the kernel that rounds fp32 operands in its registers
     same = winograd2x2_conv(gpu(ti, dev), gpu(w, dev), precision="bf16").cpu().numpy()
     assert rel_max(got, same) <= TOL

@@ -406,9 +406,12 @@ def test_forward_pair_replays_in_a_hip_graph(dev):
 
 @pytest.mark.parametrize("shape", [(3, 3, 3, 32, 32), (2, 4, 4, 5, 7), (8, 9, 9, 128, 72), (16, 14, 14, 128, 128),
                                    (1, 5, 7, 48, 20)])
-@pytest.mark.parametrize("parts", ["affine", "residual", "both"])
+@pytest.mark.parametrize("parts", ["affine", "residual", "both", "both_relu"])
 def test_conv_epilogue(oracle, dev, shape, parts):
-    # Output = fmaf(conv, scale, shift) + residual inside the stores, on every kernel the launcher picks.
+    # Output = fmaf(conv, scale, shift) + residual (or + relu(residual)) inside the stores, on every kernel the
+    # launcher picks.
+    relu_res = parts == "both_relu"
+    parts = "both" if relu_res else parts
     _, conv = ops()
     B, nH, nW, C, K = shape
     ti, w = conv_inputs(shape, 21)
@@ -422,7 +425,9 @@ def test_conv_epilogue(oracle, dev, shape, parts):
         kw.update(scale=gpu(scale, dev), shift=gpu(shift, dev))
         want = oracle.affine(want, scale, shift)
     if parts in ("residual", "both"):
-        kw.update(residual=gpu(res, dev))
+        kw.update(residual=gpu(res, dev), residual_relu=relu_res)
+        if relu_res:
+            res = np.maximum(res, 0)
         want = want + res
     got = conv(gpu(ti, dev), gpu(w, dev), **kw).cpu().numpy()
     # same kernel, same accumulators: the epilogue arithmetic itself is exact against the oracle's

@@ -73,12 +73,12 @@ def _forward_against_oracle_path(oracle, precision, tol, batch, size, check_unfo
             t = oracle.round_bf16(t)
         return torch.from_numpy(t)
 
-    def cpu_conv_forward(self, x, affine=None, residual=None):
+    def cpu_conv_forward(self, x, affine=None, residual=None, residual_relu=False):
         y = oracle.conv(x.numpy(), self.masked_weight().numpy(), acc64=True)
         if affine is not None:
             y = oracle.affine(y, affine[0].detach().numpy(), affine[1].detach().numpy())
         if residual is not None:
-            y = y + residual.numpy()
+            y = y + (np.maximum(residual.numpy(), 0) if residual_relu else residual.numpy())
         return torch.from_numpy(y)
 
     orig_imtrans, orig_forward = resnet18_var.WinogradImTrans, winograd_conv.WinogradConv.forward
