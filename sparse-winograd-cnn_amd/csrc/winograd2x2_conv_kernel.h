@@ -513,7 +513,10 @@ constexpr int async_lds_bytes()
 // output columns.
 // BF16 (forward only): the operands are rounded to bf16 (round-to-nearest-even, v_cvt_pk_bf16_f32) after they are
 // read from LDS and multiplied with v_mfma_f32_32x32x16_bf16; accumulation, fold and stores stay fp32.
-template <typename Cfg, int NSTAGE, bool BF16, int MODE>
+// NPOS: how many of the 16 positions (planes of TI, Wt and, in dgrad mode, Out) the call walks, starting at the
+// planes the three pointers point to.  The forward fold needs all 16; the products of the data gradient are
+// independent, so its launcher may deal groups of positions to different workgroups.
+template <typename Cfg, int NSTAGE, bool BF16, int MODE, int NPOS = 16>
 __device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, const float *__restrict__ Wt,
                                                float *__restrict__ Out, size_t M, int R, int N, int nW, const size_t m0,
                                                const int n0, const unsigned rows_valid, const int wm0, const int wn0,
@@ -541,6 +544,7 @@ __device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, con
     static_assert((BM * CH) % 64 == 0 && (BK * BN / 4) % 64 == 0, "tiles are whole wave-wide copies");
     static_assert((NSTAGE - 2) * LPS + (DGRAD ? TM * TN * Cfg::REGS : 0) < 64, "vmcnt range");
     static_assert(!DGRAD || NSTAGE <= 3, "the wait below allows for the stores of one earlier step");
+    static_assert(NPOS == 16 || (DGRAD && NPOS >= 1 && 16 % NPOS == 0), "the output transform folds all 16 positions");
 
     static_assert(NSTAGE * STAGE_FLOATS * 4 == async_lds_bytes<Cfg, NSTAGE, MODE>(), "launcher and kernel agree on the LDS size");
     extern __shared__ __attribute__((aligned(1024))) float smem[];  // async_lds_bytes<Cfg, NSTAGE, MODE>() bytes
@@ -629,7 +633,7 @@ __device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, con
             kc_next = 0;
             a_next += a_wrap;
             b_next += b_wrap;
-            if (++pos_next == 16) {
+            if (++pos_next == NPOS) {
                 pos_next = 0;
                 a_next = TI + m0 * R;
                 b_next = Wt;
@@ -884,14 +888,14 @@ __device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, con
 
     // The position loop is unrolled at compile time so that the signs of the output transform
     // are constants (a run-time loop over position pairs with branched folds measured 6 % slower).
-    static_for<16>([&](auto pos_tag) {
+    static_for<NPOS>([&](auto pos_tag) {
         constexpr int pos = decltype(pos_tag)::value;
         step(P[pos & 1], P[(pos & 1) ^ 1], std::true_type{}, std::integral_constant<int, pos - 1>{});
         for (int kc = 1; kc < nkc; ++kc)
             step(P[pos & 1], P[(pos & 1) ^ 1], std::false_type{}, std::integral_constant<int, -1>{});
     });
 #pragma unroll
-    for (int e = 0; e < NE; ++e) finish_unit(P[1], 15, e);
+    for (int e = 0; e < NE; ++e) finish_unit(P[(NPOS - 1) & 1], NPOS - 1, e);
 
     // The surplus copies must have landed before this workgroup's LDS can be handed on.
     wait_vmcnt<0>();
@@ -923,18 +927,24 @@ __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OC
 // Data gradient: dTI [16][M][C] from dP [16][M][K] and W [16][C][K]: dTI_i = dP_i . W_i^T.
 // Requirements checked by the launcher: K % BK == 0 (the reduction), dP and W 16-byte aligned, tile offsets
 // below 2^31 bytes.  Rows beyond M and columns beyond C are clamped on load and never stored.
-template <typename Cfg, int NSTAGE>
+// A workgroup owns one tile of NPOS consecutive planes: grid.x = (16 / NPOS) * tiles_m * tiles_n, the position
+// group slowest, so that the workgroups running at the same time work on neighbouring rows of the same planes.
+template <typename Cfg, int NSTAGE, int NPOS = 16>
 __global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_dgrad_async_kernel(
     const float *__restrict__ dP, const float *__restrict__ Wt, float *__restrict__ dTI, size_t M, int C, int K,
-    unsigned tiles_n, unsigned rows_per_wg)
+    unsigned tiles_m, unsigned tiles_n, unsigned rows_per_wg)
 {
     const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
-    const size_t m0 = static_cast<size_t>(lid / tiles_n) * rows_per_wg;
-    const int n0 = static_cast<int>(lid % tiles_n) * Cfg::BN;
+    const unsigned per_group = tiles_m * tiles_n;
+    const size_t pos0 = static_cast<size_t>(lid / per_group) * NPOS;
+    const unsigned tile = lid % per_group;
+    const size_t m0 = static_cast<size_t>(tile / tiles_n) * rows_per_wg;
+    const int n0 = static_cast<int>(tile % tiles_n) * Cfg::BN;
     const unsigned rows_valid = static_cast<unsigned>(M - m0 < rows_per_wg ? M - m0 : rows_per_wg);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same for the whole wave: scalar
     const int wm0 = (wave / Cfg::WGN) * Cfg::WM, wn0 = (wave % Cfg::WGN) * Cfg::WN;
-    conv_ring_body<Cfg, NSTAGE, false, RING_DGRAD>(dP, Wt, dTI, M, K, C, 0, m0, n0, rows_valid, wm0, wn0, ConvEpilogue());
+    conv_ring_body<Cfg, NSTAGE, false, RING_DGRAD, NPOS>(dP + pos0 * M * K, Wt + pos0 * C * K, dTI + pos0 * M * C, M, K, C, 0,
+                                                         m0, n0, rows_valid, wm0, wn0, ConvEpilogue());
 }
 
 }  // namespace

@@ -360,40 +360,37 @@ int gemm16_plain(const float *A, const float *Bm, float *Out, size_t P, int Q, s
     return check_launch();
 }
 
-// dTI [16][M][C] = dP [16][M][K] . W [16][C][K]^T on the ring kernel, in the tiling the forward launcher would
-// give a call with these extents (rows M, reduction K, columns C).  SWC_ERR_UNSUPPORTED when no ring tiling
-// takes the shapes.
-template <typename Cfg>
-int launch_dgrad(const float *dP, const float *W, float *dTI, size_t M, int C, int K, size_t rows_per_wg, hipStream_t s)
-{
-    constexpr int kStages = 2;  // a third ring slot (stores waited for a step later) measured 3 % slower
-    constexpr int lds_bytes = async_lds_bytes<Cfg, kStages, RING_DGRAD>();
-    static_assert(lds_bytes <= 160 * 1024, "a CU has 160 KiB of LDS");
-    struct Tag {};
-    const int st = raise_lds_limit<Tag>(reinterpret_cast<const void *>(conv_dgrad_async_kernel<Cfg, kStages>), lds_bytes);
-    if (st != SWC_OK) return st;
-    // Whole MFMA tiles per workgroup, so that only the last row group has a ragged tile (its waves fall back to
-    // waiting for all of their memory operations at every step).
-    rows_per_wg = (rows_per_wg + Cfg::MF - 1) / Cfg::MF * Cfg::MF;
-    const size_t tiles_m = (M + rows_per_wg - 1) / rows_per_wg;
-    const size_t tiles_n = (static_cast<size_t>(C) + Cfg::BN - 1) / Cfg::BN;
-    if (tiles_m * tiles_n >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
-    conv_dgrad_async_kernel<Cfg, kStages><<<dim3(static_cast<unsigned>(tiles_m * tiles_n)), dim3(Cfg::NT), lds_bytes, s>>>(
-        dP, W, dTI, M, C, K, static_cast<unsigned>(tiles_n), static_cast<unsigned>(rows_per_wg));
-    return check_launch();
-}
+// dTI [16][M][C] = dP [16][M][K] . W [16][C][K]^T on the ring kernel.  The 16 products are independent, so
+// the grid is (pairs of positions) x (64x64 tiles): eight times the workgroups of the forward pass, each an
+// eighth as long as one that walks all 16 positions, four resident per SIMD (the product accumulators are all the
+// registers a wave needs here).  Short workgroups at different points of their loops overlap each other's
+// waits and product stores, and the tile count no longer has to divide by the CU count.  Measured against
+// the forward pass's tilings walking all 16 positions (us, dense operands): 28x28x128 at batch 64 67.7 (tall16
+// 76.3), at batch 128 146.7 (152.5); 14x14x256 at batch 64 67.8 (short16 78.9); 56x56x64 87.9 (93.4);
+// 7x7x512 77.1 (short16 95.6).  One, two or four positions per workgroup, two to four waves per SIMD and 128-row
+// or 128-column tiles were within 5 % of this on some shapes and 10-20 % slower on others.
+// SWC_ERR_UNSUPPORTED when the ring kernel does not take the shapes (K % 32, alignment, 32-bit offsets).
+using DgradTile = ConvCfg<64, 64, 32, 2, 2, 4>;
+constexpr int kDgradPositions = 2;
 
 int dgrad_own(const float *dP, const float *W, float *dTI, size_t M, int C, int K, hipStream_t s)
 {
     // 32-bit offsets: elements within a workgroup's rows of a plane, bytes within a position's weights
-    if (static_cast<size_t>(112) * C >= (1ull << 30) || static_cast<size_t>(C) * K >= (1ull << 30)) return SWC_ERR_UNSUPPORTED;
-    const TilingChoice pick = choose_tiling(dP, W, M, K, C, false, false);
-    switch (pick.tiling) {
-        case TILING_TALL16: return launch_dgrad<Tall>(dP, W, dTI, M, C, K, pick.rows_per_wg, s);
-        case TILING_SHORT16: return launch_dgrad<Short>(dP, W, dTI, M, C, K, pick.rows_per_wg, s);
-        case TILING_RING32: return launch_dgrad<Tile32>(dP, W, dTI, M, C, K, Tile32::BM, s);
-        default: return SWC_ERR_UNSUPPORTED;
-    }
+    if (static_cast<size_t>(DgradTile::BM) * C >= (1ull << 30) || static_cast<size_t>(C) * K >= (1ull << 30))
+        return SWC_ERR_UNSUPPORTED;
+    if (!ring_eligible<DgradTile>(dP, W, K, C, false)) return SWC_ERR_UNSUPPORTED;
+    constexpr int kStages = 2;  // a third ring slot (stores waited for a step later) measured no faster
+    constexpr int lds_bytes = async_lds_bytes<DgradTile, kStages, RING_DGRAD>();
+    static_assert(lds_bytes <= 64 * 1024, "below the default dynamic LDS limit");
+    const size_t tiles_m = (M + DgradTile::BM - 1) / DgradTile::BM;
+    const size_t tiles_n = (static_cast<size_t>(C) + DgradTile::BN - 1) / DgradTile::BN;
+    const size_t groups = 16 / kDgradPositions;
+    if (groups * tiles_m * tiles_n >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
+    conv_dgrad_async_kernel<DgradTile, kStages, kDgradPositions>
+        <<<dim3(static_cast<unsigned>(groups * tiles_m * tiles_n)), dim3(DgradTile::NT), lds_bytes, s>>>(
+            dP, W, dTI, M, C, K, static_cast<unsigned>(tiles_m), static_cast<unsigned>(tiles_n),
+            static_cast<unsigned>(DgradTile::BM));
+    return check_launch();
 }
 
 // dW through the split-reduction kernel.  The partial tiles of the S row splits are parked in the
