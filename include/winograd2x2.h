@@ -236,6 +236,18 @@ SWC_API int swc_winograd2x2_relu_conv_bf16(const float *Input, const float *InSc
                                    const float *OutShift, const float *Residual, int C, int B, int H, int W,
                                    int K, int pad_h, int pad_w, int relu, swc_stream_t stream);
 
+/*
+ * 1x1 convolution over NHWC pixels: Output [M,K] = Input [M,C] . Weight [K,C]^T, M = B*H*W, fp32.
+ * No counterpart among the reference's custom ops: its model takes the shortcut of the first unit of every stage
+ * through tensorpack's Conv2D (`Conv2D('res2a_1', l, 64, 1, ...)`, ResNet-18-var/imagenet-resnet-transWino-prune.py:127,
+ * :152, :177, :202).  Here it runs on the kernel of the convolution's data gradient (one of its 16 products has
+ * exactly this form), which reads and writes each byte once where the library GEMM PyTorch picks for these
+ * skinny shapes takes 2-6 times as long.  Needs C % 32 == 0 and 16-byte aligned operands; returns
+ * SWC_ERR_UNSUPPORTED otherwise (use any GEMM).
+ */
+SWC_API int swc_winograd2x2_pointwise_conv(const float *Input, const float *Weight, float *Output, int C, long long M,
+                                           int K, swc_stream_t stream);
+
 /* ---------------------------------------------------------------------------
  * Backward ops.
  * ------------------------------------------------------------------------- */

@@ -594,6 +594,31 @@ int imtrans_grad_entry(const float *TransIm_grad, const float *relu_mask_source,
 }  // namespace
 }  // namespace swc
 
+// Out [M][K] = Input [M][C] . Weight [K][C]^T: a 1x1 convolution over NHWC pixels.  It is one position of the data
+// gradient's product with the roles renamed, so it runs on the same kernel, one plane per workgroup.
+extern "C" int swc_winograd2x2_pointwise_conv(const float *Input, const float *Weight, float *Output, int C, long long M,
+                                              int K, swc_stream_t stream)
+{
+    using namespace swc;
+    if (Input == nullptr || Weight == nullptr || Output == nullptr) return SWC_ERR_NULL_POINTER;
+    if (C <= 0 || K <= 0 || M <= 0 || M >= (1ll << 31)) return SWC_ERR_BAD_DIMS;
+    // reduction over C in whole 32-index steps, 16-byte copies, 32-bit offsets within a tile's rows and the weights
+    if (static_cast<size_t>(DgradTile::BM) * K >= (1ull << 30) || static_cast<size_t>(C) * K >= (1ull << 30) ||
+        !ring_eligible<DgradTile>(Input, Weight, C, K, false))
+        return SWC_ERR_UNSUPPORTED;
+    constexpr int kStages = 2;
+    constexpr int lds_bytes = async_lds_bytes<DgradTile, kStages, RING_DGRAD>();
+    const size_t rows = static_cast<size_t>(M);
+    const size_t tiles_m = (rows + DgradTile::BM - 1) / DgradTile::BM;
+    const size_t tiles_n = (static_cast<size_t>(K) + DgradTile::BN - 1) / DgradTile::BN;
+    if (tiles_m * tiles_n >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
+    conv_dgrad_async_kernel<DgradTile, kStages, 1>
+        <<<dim3(static_cast<unsigned>(tiles_m * tiles_n)), dim3(DgradTile::NT), lds_bytes, static_cast<hipStream_t>(stream)>>>(
+            Input, Weight, Output, rows, K, C, static_cast<unsigned>(tiles_m), static_cast<unsigned>(tiles_n),
+            static_cast<unsigned>(DgradTile::BM));
+    return check_launch();
+}
+
 extern "C" int swc_winograd2x2_imtrans_grad(const float *TransIm_grad, const float *relu_mask_source, float *Input_grad,
                                             int C, int B, int H, int W, int pad_h, int pad_w, swc_stream_t stream)
 {

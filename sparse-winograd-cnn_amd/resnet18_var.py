@@ -23,6 +23,7 @@ import torch
 import torch.nn.functional as F
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+import swc_hip  # noqa: E402
 from winograd_conv import WinogradConv  # noqa: E402
 from winograd_imtrans import WinogradImTrans  # noqa: E402
 
@@ -84,17 +85,32 @@ def _conv_bn_folded(conv, bn):
 
 def _shortcut_folded(conv, bn, bn_out):
     """The 1x1 shortcut conv + its BatchNorm, for a branch whose last convolution applies ``bn_out`` and adds
-    the shortcut in its stores: returns (Wt [Cin,Cout], scale, shift) such that
-    ``branch*scale + shift + x_nhwc @ Wt == bn_out(branch) + bn(conv(x))``.  A 1x1 convolution over NHWC data is
+    the shortcut in its stores: returns (W [Cout,Cin], scale, shift) such that
+    ``branch*scale + shift + x_nhwc @ W.T == bn_out(branch) + bn(conv(x))``.  A 1x1 convolution over NHWC data is
     one matrix product, and its bias joins the shift the kernel adds anyway.  Cached like _conv_bn_folded."""
     w1, b1 = _conv_bn_folded(conv, bn)
     scale, shift = _bn_affine(bn_out)
     key = (conv._swc_folded[0], bn_out._swc_affine[0])
     cached = getattr(conv, "_swc_shortcut", None)
     if cached is None or cached[0] != key:
-        cached = (key, w1.view(w1.shape[0], w1.shape[1]).t().contiguous(), scale, (shift + b1).contiguous())
+        cached = (key, w1.view(w1.shape[0], w1.shape[1]).contiguous(), scale, (shift + b1).contiguous())
         conv._swc_shortcut = cached
     return cached[1], cached[2], cached[3]
+
+
+def pointwise_conv(x, w):
+    """x [B,H,W,C] NHWC, w [K,C] -> [B,H,W,K]: a 1x1 convolution.  On the GPU it runs on the library's kernel
+    (``swc_winograd2x2_pointwise_conv``) where that takes the shape (C % 32 == 0), else as a matrix product."""
+    B, H, W, C = x.shape
+    if x.is_cuda and x.dtype == torch.float32 and w.dtype == torch.float32 and x.is_contiguous() and w.is_contiguous():
+        out = torch.empty((B, H, W, w.shape[0]), dtype=torch.float32, device=x.device)
+        with swc_hip.on_device(x.device) as stream:
+            st = swc_hip.lib().swc_winograd2x2_pointwise_conv(x.data_ptr(), w.data_ptr(), out.data_ptr(), C, B * H * W,
+                                                              w.shape[0], stream)
+        if st != swc_hip.SWC_ERR_UNSUPPORTED:
+            swc_hip.check(st, "pointwise_conv")
+            return out
+    return torch.mm(x.reshape(-1, C), w.t()).view(B, H, W, w.shape[0])
 
 
 def _to_nhwc(x):   # NCHW tensor in channels_last memory -> contiguous [B,H,W,C] view
@@ -143,11 +159,16 @@ class WinogradUnit(torch.nn.Module):
     def forward(self, x):
         out_affine = None
         if self.shortcut:
-            s = torch.relu(self.bn_pre(x)) if self.bn_pre is not None else torch.relu(x)
+            if self.bn_pre is not None and self.fold_bn:
+                # BNReLU as x*scale + shift and an in-place ReLU: two elementwise passes instead of the library
+                # BatchNorm's slower one plus a ReLU that allocates
+                a, b = _bn_affine(self.bn_pre)
+                s = torch.addcmul(b.view(1, -1, 1, 1), x, a.view(1, -1, 1, 1)).relu_()
+            else:
+                s = torch.relu(self.bn_pre(x)) if self.bn_pre is not None else torch.relu(x)
             if self.fold_bn:
-                wt, scale, shift = _shortcut_folded(self.conv1, self.bn1, self.bn2c)
-                s = _to_nhwc(s)
-                sc = torch.mm(s.view(-1, s.shape[3]), wt).view(s.shape[0], s.shape[1], s.shape[2], wt.shape[1])
+                w1, scale, shift = _shortcut_folded(self.conv1, self.bn1, self.bn2c)
+                sc = pointwise_conv(_to_nhwc(s), w1)
                 out_affine = (scale, shift)
             else:
                 sc = self.bn1(self.conv1(s))

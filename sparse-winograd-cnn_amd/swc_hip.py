@@ -30,7 +30,7 @@ C_SYMBOLS = (
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
     "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad", "swc_winograd2x2_imtrans_grad_relu_input",
-    "swc_winograd2x2_relu_conv",
+    "swc_winograd2x2_relu_conv", "swc_winograd2x2_pointwise_conv",
 )
 # The two C++-linkage launchers with the reference's exact signatures (Itanium mangling).
 CXX_SYMBOLS = (
@@ -78,6 +78,8 @@ def lib():
         L.swc_winograd2x2_conv_last_kernel.argtypes = []
         L.swc_winograd2x2_conv_force_tiling.restype = i32
         L.swc_winograd2x2_conv_force_tiling.argtypes = [ctypes.c_char_p]
+        L.swc_winograd2x2_pointwise_conv.restype = i32
+        L.swc_winograd2x2_pointwise_conv.argtypes = [fp] * 3 + [i32, ctypes.c_longlong, i32, vp]
         L.swc_winograd2x2_conv_grad_static.restype = i32
         L.swc_winograd2x2_conv_grad_static.argtypes = [fp] * 5 + [i32] * 7 + [vp]
         L.swc_winograd2x2_imtrans.restype = i32

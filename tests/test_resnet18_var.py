@@ -32,6 +32,33 @@ PRECISIONS = [("fp32", 1e-3), ("bf16", 5e-2), ("bf16_stored", 5e-2)]
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(2, 7, 9, 64, 64), (1, 5, 5, 32, 40), (3, 14, 14, 128, 256), (1, 3, 3, 96, 20),
+                                   (2, 4, 4, 48, 64)])
+def test_pointwise_conv(shape):
+    # The model's 1x1 shortcut convolutions (imagenet-resnet-transWino-prune.py:127,152,177,202) as a product over
+    # NHWC pixels: against float64 numpy, exact on small integers; C = 48 is not taken by the kernel and falls back.
+    import resnet18_var
+    import swc_hip
+    B, H, W, C, K = shape
+    rng = np.random.default_rng(77)
+    dev = torch.device("cuda:0")
+    x = rng.standard_normal((B, H, W, C)).astype(np.float32)
+    w = rng.standard_normal((K, C)).astype(np.float32)
+    got = resnet18_var.pointwise_conv(torch.from_numpy(x).to(dev), torch.from_numpy(w).to(dev)).cpu().numpy()
+    want = x.astype(np.float64).reshape(-1, C) @ w.astype(np.float64).T
+    assert got.shape == (B, H, W, K)
+    assert rel_max(got.reshape(-1, K), want) <= 1e-5
+    xi = rng.integers(-4, 5, size=x.shape).astype(np.float32)
+    wi = rng.integers(-4, 5, size=w.shape).astype(np.float32)
+    goti = resnet18_var.pointwise_conv(torch.from_numpy(xi).to(dev), torch.from_numpy(wi).to(dev)).cpu().numpy()
+    assert np.array_equal(goti.reshape(-1, K), xi.reshape(-1, C) @ wi.T)
+    out = torch.empty(B * H * W * K, device=dev)
+    st = swc_hip.lib().swc_winograd2x2_pointwise_conv(torch.from_numpy(x).to(dev).data_ptr(), torch.from_numpy(w).to(dev).data_ptr(),
+                                                      out.data_ptr(), C, B * H * W, K, torch.cuda.current_stream().cuda_stream)
+    assert st == (swc_hip.SWC_ERR_UNSUPPORTED if C % 32 else 0)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("precision,tol", PRECISIONS)
 def test_forward_matches_oracle_path(oracle, precision, tol):
     _forward_against_oracle_path(oracle, precision, tol, batch=2, size=64, check_unfolded=True)
