@@ -169,9 +169,13 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
         return SWC_ERR_UNSUPPORTED;
     const size_t tiles_n = (static_cast<size_t>(K) + HB_BN - 1) / HB_BN;
     // Rows per workgroup: the workgroup count rounded up to a multiple of the CU count, as for the fp32
-    // tilings (49 to 64 rows; conv2: 26.7 vs 28.8 us).
+    // tilings (49 to 64 rows; conv2: 26.7 vs 28.8 us) -- unless the weights fill an L2 or more.  Every row group
+    // walks all of the weights of its columns, and what does not stay in the XCD's L2 comes from the Infinity
+    // Cache again for each of them: then the tallest tile (fewest row groups) and the deeper ring (a step more of
+    // latency covered) win: 14x14 at batch 128, 512 -> 512: 96 us against 124 us, 256 -> 512: 57 against 66.
     const size_t cus = device_cus();
-    const size_t rows = balanced_rows<HbStoreCfg>(M, tiles_n, cus);
+    const bool weights_beyond_l2 = static_cast<size_t>(16) * C * K * 2 >= device_l2_bytes();
+    const size_t rows = weights_beyond_l2 ? static_cast<size_t>(HB_BM) : balanced_rows<HbStoreCfg>(M, tiles_n, cus);
     const size_t tiles_m = (M + rows - 1) / rows;
     if (tiles_m * tiles_n >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
     ConvEpilogue ep;
@@ -183,7 +187,7 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
     // More resident workgroups hide more of each other's waits once there are enough of them to go round
     // (conv3: 18.7 vs 19.6 us); a grid that leaves CUs with one workgroup does better with the deeper
     // ring (conv4b: 30.8 vs 34.2 us).
-    if (tiles_m * tiles_n > cus) {
+    if (tiles_m * tiles_n > cus && !weights_beyond_l2) {
         note_conv_kernel("stored-ring3");
         return launch_bf16_stored<Wide>(Input16, Weight16t, Output, M, C, K, nH, nW, rows, tiles_n, ep, s);
     }

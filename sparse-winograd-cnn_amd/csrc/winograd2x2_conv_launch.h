@@ -24,6 +24,21 @@ inline size_t device_cus()
     return static_cast<size_t>(cus[dev]);
 }
 
+// Bytes of one L2 (MI355X: 4 MiB per XCD, eight of them), read once per device and host thread.
+inline size_t device_l2_bytes()
+{
+    constexpr int kMaxDevices = 64;
+    static thread_local int l2[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 4u << 20;
+    if (l2[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeL2CacheSize, dev) != hipSuccess || n <= 0) n = 4 << 20;
+        l2[dev] = n;
+    }
+    return static_cast<size_t>(l2[dev]);
+}
+
 namespace {
 
 // 32x32 MFMAs, wave tile 32x32: the fewest LDS reads per MFMA; its results are bit-identical to
