@@ -44,11 +44,13 @@ SWC_API const char *swc_version(void);
  * thread's last swc_winograd2x2_conv / _conv_bf16 / _conv_epilogue / _conv_bf16in call launched ("" before the
  * first): "sync" (any shape and alignment), "ring32" / "ring16" (64x64 tiles, 32- / 16-channel steps),
  * "tall16" / "short16" (row groups of up to 112 / 32 rows, dealt evenly over the CUs); for bf16-stored operands
- * "stored-ring3" / "stored-ring4" (64x64 tiles, 3- / 4-deep copy ring).  Which one runs depends only on the
- * shapes and pointer alignment; all give the same results to within the order of the reduction over C. */
+ * "stored-ring3" / "stored-ring4" (64x64 tiles, 3- / 4-deep copy ring) / "stored-split" (small grids: the 16
+ * positions of a tile split over two groups of waves, whose partial sums are added at the end).  Which one runs
+ * depends only on the shapes, pointer alignment and the device's CU count and L2 size; all give the same results
+ * to within the order of the fp32 summations. */
 SWC_API const char *swc_winograd2x2_conv_last_kernel(void);
 /* Diagnostic with no counterpart in the reference, for benchmarks and tests that compare the tilings: makes
- * the calling thread's later swc_winograd2x2_conv calls (and the data-gradient GEMM of swc_winograd2x2_conv_grad)
+ * the calling thread's later swc_winograd2x2_conv calls
  * use the named kernel ("ring32", "ring16", "tall16", "short16", "sync") where the shapes allow it and "sync"
  * where they do not; NULL or "" gives the choice back to the launcher.  Returns SWC_ERR_UNSUPPORTED for an
  * unknown name. */

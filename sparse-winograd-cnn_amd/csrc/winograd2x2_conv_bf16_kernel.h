@@ -39,8 +39,15 @@ struct HbCfg {
 };
 
 // Requires C % BK == 0 and 16-byte aligned TI16 / Wt16.  M < 2^31.  grid.x = ceil(M / rows_per_wg) * tiles_n.
-template <typename Cfg>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_bf16_stored_kernel(
+//
+// GROUPS = 2: a workgroup is two groups of four waves that share the tile and split its 16 positions, 0-7 and
+// 8-15, each group with its own ring; at the end the second group hands its four partial output tiles to the first
+// through LDS, which adds them to its own and stores.  For grids that leave a CU with one workgroup: the time
+// of such a launch is one workgroup's chain of dependent steps (wait, barrier, copies, LDS reads, four MFMAs), and
+// two chains of half the length run side by side on the same SIMDs.  The sum of the transform is then taken as
+// (positions 0-7) + (positions 8-15) instead of in one ascending chain.  Needs 2*LDS_BYTES of LDS.
+template <typename Cfg, int GROUPS = 1>
+__global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_bf16_stored_kernel(
     const unsigned short *__restrict__ TI16, const unsigned short *__restrict__ Wt16, float *__restrict__ Out, size_t M,
     int C, int K, int nH, int nW, unsigned tiles_n, unsigned rows_per_wg, ConvEpilogue ep)
 {
@@ -55,11 +62,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
     const unsigned rows_valid = static_cast<unsigned>(M - m0 < rows_per_wg ? M - m0 : rows_per_wg);
     const unsigned cols_valid = static_cast<unsigned>(K - n0 < HB_BN ? K - n0 : HB_BN);
 
+    static_assert(GROUPS == 1 || GROUPS == 2, "one or two groups of four waves");
+    constexpr int NPOS = 16 / GROUPS;  // positions per group
     const int tid = threadIdx.x, lane = tid & 63;
-    const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const unsigned wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const unsigned group = wave_wg >> 2, wave = wave_wg & 3;  // wave: index within the group
     const int li = lane & 31, lg = lane >> 5;
     const int wm0 = static_cast<int>(wave >> 1) * 32, wn0 = static_cast<int>(wave & 1) * 32;
     const int nkc = C / BK;
+    unsigned char *const smem_g = smem_b + group * Cfg::LDS_BYTES;  // this group's ring
 
     // ---- copies: wave-copy wl of a tile covers its rows RPC*wl .. RPC*wl+RPC-1 (1 KiB) ------------------
     // Rows beyond the valid ones re-read the last valid row; they only reach outputs that are never stored.
@@ -73,14 +84,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
         b_voff[q] = (rb * static_cast<unsigned>(C) + chunk * 8) * 2u;
         t_lds[q] = wl * 1024u;
     }
-    const unsigned smem_base = lds_address(smem_b);
+    const unsigned smem_base = lds_address(smem_g);
     const size_t a_pos_stride = M * static_cast<size_t>(C), b_pos_stride = static_cast<size_t>(K) * C;
-    const unsigned short *a_pos = TI16 + m0 * C, *b_pos = Wt16 + static_cast<size_t>(n0) * C;
+    // the group's first position: 0, or 8 for the second group
+    const unsigned short *const a_first = TI16 + m0 * C + group * NPOS * a_pos_stride;
+    const unsigned short *const b_first = Wt16 + static_cast<size_t>(n0) * C + group * NPOS * b_pos_stride;
+    const unsigned short *a_pos = a_first, *b_pos = b_first;
     const unsigned short *a_next = a_pos, *b_next = b_pos;
     int kc_next = 0, pos_next = 0;
     unsigned slot_next = 0;
     // Every thread issues exactly Cfg::COPIES copies per call; past the last step the walk wraps to
-    // position 0 again (copied, never read).
+    // the group's first position again (copied, never read).
     auto issue = [&]() __attribute__((always_inline)) {
         const unsigned dst = smem_base + slot_next * Cfg::STAGE_BYTES;
 #pragma unroll
@@ -90,10 +104,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
             async_copy16(reinterpret_cast<const float *>(b_next), b_voff[q], dst + Cfg::TILE_BYTES + t_lds[q]);
         if (++kc_next == nkc) {
             kc_next = 0;
-            if (++pos_next == 16) {
+            if (++pos_next == NPOS) {
                 pos_next = 0;
-                a_pos = TI16 + m0 * C;
-                b_pos = Wt16 + static_cast<size_t>(n0) * C;
+                a_pos = a_first;
+                b_pos = b_first;
             } else {
                 a_pos += a_pos_stride;
                 b_pos += b_pos_stride;
@@ -141,56 +155,83 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, C
         issue();
 #pragma unroll
         for (int h = 0; h < Cfg::NMFMA; ++h) {
-            fa[set][h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_next + a_off[h]);
-            fb[set][h] = *reinterpret_cast<const bf16x8 *>(smem_b + st_next + b_off[h]);
+            fa[set][h] = *reinterpret_cast<const bf16x8 *>(smem_g + st_next + a_off[h]);
+            fb[set][h] = *reinterpret_cast<const bf16x8 *>(smem_g + st_next + b_off[h]);
         }
         st_next = st_next + Cfg::STAGE_BYTES == Cfg::LDS_BYTES ? 0 : st_next + Cfg::STAGE_BYTES;
     };
     fetch(0);
 
-    static_for<16>([&](auto pos_tag) {
-        constexpr int pos = decltype(pos_tag)::value;
-        floatx16 P = {};
-        auto mfmas = [&](int set) __attribute__((always_inline)) {
-#pragma unroll
-            for (int h = 0; h < Cfg::NMFMA; ++h) P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][h], fb[set][h], P, 0, 0, 0);
-        };
-        // A position starts with its first step's operands in set 0.  Steps go in pairs so that the set
-        // indices are compile-time constants (the sets must stay in registers); an odd last step moves
-        // the prefetched set 1 into set 0.  Past the very last step the fetch reads the wrapped-around
-        // copy, which is never used.
-        int kc = 0;
-#pragma nounroll
-        for (; kc + 1 < nkc; kc += 2) {
-            fetch(1);
-            mfmas(0);
-            fetch(0);
-            mfmas(1);
-        }
-        if (kc < nkc) {
-            fetch(1);
-            mfmas(0);
-#pragma unroll
-            for (int h = 0; h < Cfg::NMFMA; ++h) {
-                fa[0][h] = fa[1][h];
-                fb[0][h] = fb[1][h];
+    auto positions = [&](auto first_tag) __attribute__((always_inline)) {
+        static_for<NPOS>([&](auto pos_tag) {
+            constexpr int pos = decltype(first_tag)::value + decltype(pos_tag)::value;
+            floatx16 P = {};
+            auto mfmas = [&](int set) __attribute__((always_inline)) {
+    #pragma unroll
+                for (int h = 0; h < Cfg::NMFMA; ++h) P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][h], fb[set][h], P, 0, 0, 0);
+            };
+            // A position starts with its first step's operands in set 0.  Steps go in pairs so that the set
+            // indices are compile-time constants (the sets must stay in registers); an odd last step moves
+            // the prefetched set 1 into set 0.  Past the very last step the fetch reads the wrapped-around
+            // copy, which is never used.
+            int kc = 0;
+    #pragma nounroll
+            for (; kc + 1 < nkc; kc += 2) {
+                fetch(1);
+                mfmas(0);
+                fetch(0);
+                mfmas(1);
             }
-        }
-        // fold P_pos into the running output tiles, ascending pos (winograd2x2_conv_cuda.cu.cc:39-46)
-        constexpr unsigned long long plus = kPlus, minus = kMinus;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if ((plus >> (4 * pos + j)) & 1ull)
-                Y[j][0][0] += P;
-            else if ((minus >> (4 * pos + j)) & 1ull)
-                Y[j][0][0] -= P;
-            // pins the update here: otherwise the compiler defers all the adds to the end and keeps the
-            // 16 product tiles alive instead of the 4 sums
-            asm volatile("" : "+v"(Y[j][0][0]));
-        }
-    });
+            if (kc < nkc) {
+                fetch(1);
+                mfmas(0);
+    #pragma unroll
+                for (int h = 0; h < Cfg::NMFMA; ++h) {
+                    fa[0][h] = fa[1][h];
+                    fb[0][h] = fb[1][h];
+                }
+            }
+            // fold P_pos into the running output tiles, ascending pos (winograd2x2_conv_cuda.cu.cc:39-46)
+            constexpr unsigned long long plus = kPlus, minus = kMinus;
+    #pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if ((plus >> (4 * pos + j)) & 1ull)
+                    Y[j][0][0] += P;
+                else if ((minus >> (4 * pos + j)) & 1ull)
+                    Y[j][0][0] -= P;
+                // pins the update here: otherwise the compiler defers all the adds to the end and keeps the
+                // 16 product tiles alive instead of the 4 sums
+                asm volatile("" : "+v"(Y[j][0][0]));
+            }
+        });
+    };
+    if (GROUPS == 1 || group == 0)
+        positions(std::integral_constant<int, 0>{});
+    else
+        positions(std::integral_constant<int, 16 - NPOS>{});
     wait_vmcnt<0>();  // the surplus copies must land before the workgroup's LDS is handed on
 
+    if constexpr (GROUPS == 2) {
+        // The second group's partial sums go through LDS, [j][register][thread of the group] (64 KiB: the rings are
+        // idle by now), and are added to the first group's, which then stores alone.
+        static_assert(2 * Cfg::LDS_BYTES >= 4 * 16 * 256 * 4, "the rings hold the four partial tiles");
+        float *const xch = reinterpret_cast<float *>(smem_b);
+        const int t = tid & 255;
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_s_barrier();  // every wave has finished reading its ring
+        if (group == 1) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) xch[(j * 16 + r) * 256 + t] = Y[j][0][0][r];
+        }
+        __syncthreads();
+        if (group == 1) return;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) Y[j][0][0][r] += xch[(j * 16 + r) * 256 + t];
+    }
     store_output<HbStoreCfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
 }
 

@@ -86,6 +86,10 @@ def test_conv_over_bf16_operands(oracle, dev, shape):
     # the same values as the kernel that rounds fp32 operands in its registers
     same = winograd2x2_conv(gpu(ti, dev), gpu(w, dev), precision="bf16").cpu().numpy()
     assert rel_max(got, same) <= TOL
+    # these grids leave every CU with one workgroup at most: two groups of waves split the positions
+    import swc_hip
+    winograd2x2_conv(ti_gpu, gpu(w, dev))
+    assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() == b"stored-split"
 
 
 def test_unsupported_channel_count_is_reported(dev):

@@ -179,3 +179,6 @@ def test_layers_at_batch_128(oracle, hw, C, K, precision):
         assert rel_max(y[sl].cpu().numpy(), want) <= 1e-4, (kernel, sl)
     if precision == "fp32":
         assert kernel != "sync", kernel   # every model shape runs on one of the copy-ring tilings
+    if stored:
+        # more tiles than CUs at every layer; weights of 4 MiB and more (an L2) take the deeper ring
+        assert kernel == ("stored-ring4" if 16 * C * K * 2 >= (4 << 20) else "stored-ring3"), kernel
