@@ -44,9 +44,9 @@ MEASURED_TRAFFIC = {
     ("cfg3", "bf16_stored", "imtrans"): (None, (12584.0 * 2 + 50176.0) * 1024),
     ("cfg2", "bf16_stored", "conv"): ("stored-ring3", (58817.0 * 2 + 50176.0) * 1024),
     ("cfg2", "bf16_stored", "imtrans"): (None, (25128.0 * 2 + 100352.0) * 1024),
-    ("cfg4a", "bf16_stored", "conv"): ("stored-ring4", (21878.5 * 2 + 12544.0) * 1024),
+    ("cfg4a", "bf16_stored", "conv"): ("stored-split", (23787.5 * 2 + 12544.0) * 1024),
     ("cfg4a", "bf16_stored", "imtrans"): (None, (6312.0 * 2 + 25088.0) * 1024),
-    ("cfg4b", "bf16_stored", "conv"): ("stored-ring4", (45330.2 * 2 + 8192.0) * 1024),
+    ("cfg4b", "bf16_stored", "conv"): ("stored-split", (43147.5 * 2 + 8192.0) * 1024),
     ("cfg4b", "bf16_stored", "imtrans"): (None, (3176.0 * 2 + 16384.0) * 1024),
 }
 
