@@ -491,7 +491,7 @@ namespace swc {
 namespace {
 
 constexpr size_t kStaticScratchFloats = SWC_CONV_GRAD_STATIC_MAX_FLOATS;
-__device__ __align__(256) float scratch[kStaticScratchFloats];
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
 
 float *static_scratch(int *status)
 {
