@@ -8,8 +8,9 @@
 // Both operands have the reduction index (channels) as their fast axis, so both LDS tiles are
 // [64 rows][64 channels = 128 bytes = 8 chunks of 16 bytes] and an MFMA operand
 // (v_mfma_f32_32x32x16_bf16: lane (li, lg) holds 8 consecutive channels 8*lg.. of row li) is one
-// ds_read_b128 with no conversion.  Chunk c of row r is stored at slot c ^ (r % 8): the 32 lanes of
-// an operand read then spread over all banks.
+// ds_read_b128 with no conversion.  Chunk c of row r is stored at slot c ^ ((r / 2) % 8): two 128-byte rows
+// share 256 bytes of LDS, and with r % 8 rows r and r+8 of an operand read landed on the same banks (the
+// counters showed every second LDS cycle as a bank conflict; none with r / 2).
 #pragma once
 
 #include "winograd2x2_conv_kernel.h"
@@ -53,6 +54,7 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(Cf
 {
     constexpr int BK = Cfg::BK, NSTAGE = Cfg::NSTAGE, CH = Cfg::CH, RPC = Cfg::ROWS_PER_COPY, PW = Cfg::PER_WAVE;
     constexpr int ROW_BYTES = BK * 2;
+    constexpr int RPL = ROW_BYTES >= 256 ? 1 : 256 / ROW_BYTES;  // tile rows per 256 bytes of LDS (one pass over its banks)
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem_b[];
 
     const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
@@ -78,7 +80,7 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(Cf
 #pragma unroll
     for (int q = 0; q < PW; ++q) {
         const unsigned wl = wave * PW + q;
-        const unsigned row = RPC * wl + lane / CH, slot = lane % CH, chunk = slot ^ (row % CH);
+        const unsigned row = RPC * wl + lane / CH, slot = lane % CH, chunk = slot ^ ((row / RPL) % CH);
         const unsigned ra = row < rows_valid ? row : rows_valid - 1, rb = row < cols_valid ? row : cols_valid - 1;
         a_voff[q] = (ra * static_cast<unsigned>(C) + chunk * 8) * 2u;
         b_voff[q] = (rb * static_cast<unsigned>(C) + chunk * 8) * 2u;
@@ -135,8 +137,8 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(Cf
 #pragma unroll
     for (int h = 0; h < Cfg::NMFMA; ++h) {
         const unsigned ra = wm0 + li, rb = wn0 + li;
-        a_off[h] = ra * ROW_BYTES + (((2 * h + lg) ^ (ra % CH)) * 16u);
-        b_off[h] = Cfg::TILE_BYTES + rb * ROW_BYTES + (((2 * h + lg) ^ (rb % CH)) * 16u);
+        a_off[h] = ra * ROW_BYTES + (((2 * h + lg) ^ ((ra / RPL) % CH)) * 16u);
+        b_off[h] = Cfg::TILE_BYTES + rb * ROW_BYTES + (((2 * h + lg) ^ ((rb / RPL) % CH)) * 16u);
     }
     unsigned st_next = 0;  // byte offset of the ring slot whose operands are fetched next
 

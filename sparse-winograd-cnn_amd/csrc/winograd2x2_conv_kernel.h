@@ -526,6 +526,11 @@ __device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, con
     constexpr int TM = Cfg::TM, TN = Cfg::TN;
     constexpr int KS = BK / KG, CH = BK / 4, NWAVES = NT / 64;
     constexpr bool DGRAD = MODE == RING_DGRAD;
+    // Chunk j of tile row r sits at slot j ^ ((r >> SWZ) % CH).  With 32-row MFMA operands and 128-byte rows, two
+    // rows share 256 bytes of LDS and rows r and r+8 of an operand read would otherwise land on the same banks
+    // (the counters showed every second LDS cycle of the data gradient as a bank conflict); the 16-row tilings
+    // measure conflict-free as they are.
+    constexpr int SWZ = (MF == 32 && BK == 32) ? 1 : 0;
     // Copies are wave-wide: 64 lanes x 16 bytes = 1 KiB.  NAW / NBW of them make an A / B tile; every
     // wave issues the same number (NA + NB) per step so that all waves count outstanding copies alike;
     // where the tile does not divide evenly the surplus copies repeat an earlier one (same bytes twice).
@@ -565,7 +570,7 @@ __device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, con
         const unsigned wl = (q * NWAVES + wave_u) % NAW;
         const unsigned slot = wl * 64 + lane;
         unsigned row = slot / CH;
-        const unsigned chunk = (slot % CH) ^ (row % CH);
+        const unsigned chunk = (slot % CH) ^ ((row >> SWZ) % CH);
         row = row < rows_valid ? row : rows_valid - 1;
         a_voff[q] = (row * static_cast<unsigned>(R) + chunk * 4) * 4u;
         a_lds[q] = wl * 1024u;
@@ -576,7 +581,7 @@ __device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, con
         const unsigned slot = wl * 64 + lane;
         if (DGRAD) {   // B tile [BN columns][BK reduction indices], swizzled like A
             unsigned col = slot / CH;
-            const unsigned chunk = (slot % CH) ^ (col % CH);
+            const unsigned chunk = (slot % CH) ^ ((col >> SWZ) % CH);
             col = n0 + col < static_cast<unsigned>(N) ? n0 + col : static_cast<unsigned>(N) - 1;
             b_voff[q] = (col * static_cast<unsigned>(R) + chunk * 4) * 4u;
             b_lds[q] = A_FLOATS * 4 + wl * 1024u;
@@ -670,7 +675,7 @@ __device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, con
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
             const int row = wm0 + tm * MF + li;
-            a_off[k8][tm] = row * CH + ((LG * k8 + lg) ^ (row % CH));  // in 16-byte units
+            a_off[k8][tm] = row * CH + ((LG * k8 + lg) ^ ((row >> SWZ) % CH));  // in 16-byte units
         }
     // Forward: B row k sits at k*BN floats plus BPAD per 4 rows; lane group lg reads rows 4*lg + t of a group.
     constexpr int BROW4 = 4 * BN + BPAD;
@@ -682,7 +687,7 @@ __device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, con
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
                 const int col = wn0 + tn * MF + li;
-                bq_off[k8][tn] = A_FLOATS / 4 + col * CH + ((LG * k8 + lg) ^ (col % CH));
+                bq_off[k8][tn] = A_FLOATS / 4 + col * CH + ((LG * k8 + lg) ^ ((col >> SWZ) % CH));
             }
     }
 
