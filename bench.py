@@ -40,13 +40,13 @@ MEASURED_TRAFFIC = {
     ("cfg4a", "fp32", "imtrans"): (None, (6432.0 * 2 + 50176.0) * 1024),
     ("cfg4b", "fp32", "conv"): ("short16", (83452.0 * 2 + 8192.0) * 1024),       # algorithmic 58.7 MB
     ("cfg4b", "fp32", "imtrans"): (None, (3175.0 * 2 + 32768.0) * 1024),
-    ("cfg3", "bf16_stored", "conv"): ("stored-ring3", (29942.5 * 2 + 25088.0) * 1024),   # algorithmic 77.6 MB
+    ("cfg3", "bf16_stored", "conv"): ("stored-ring3", (29943.0 * 2 + 25088.0) * 1024),   # algorithmic 77.6 MB
     ("cfg3", "bf16_stored", "imtrans"): (None, (12584.0 * 2 + 50176.0) * 1024),
-    ("cfg2", "bf16_stored", "conv"): ("stored-ring3", (58817.0 * 2 + 50176.0) * 1024),
+    ("cfg2", "bf16_stored", "conv"): ("stored-ring3", (58798.7 * 2 + 50176.0) * 1024),
     ("cfg2", "bf16_stored", "imtrans"): (None, (25128.0 * 2 + 100352.0) * 1024),
-    ("cfg4a", "bf16_stored", "conv"): ("stored-split", (23787.5 * 2 + 12544.0) * 1024),
+    ("cfg4a", "bf16_stored", "conv"): ("stored-split", (23787.0 * 2 + 12544.0) * 1024),
     ("cfg4a", "bf16_stored", "imtrans"): (None, (6312.0 * 2 + 25088.0) * 1024),
-    ("cfg4b", "bf16_stored", "conv"): ("stored-split", (43147.5 * 2 + 8192.0) * 1024),
+    ("cfg4b", "bf16_stored", "conv"): ("stored-split", (43147.0 * 2 + 8192.0) * 1024),
     ("cfg4b", "bf16_stored", "imtrans"): (None, (3176.0 * 2 + 16384.0) * 1024),
 }
 
