@@ -526,11 +526,11 @@ __device__ __forceinline__ void conv_ring_body(const float *__restrict__ TI, con
     constexpr int TM = Cfg::TM, TN = Cfg::TN;
     constexpr int KS = BK / KG, CH = BK / 4, NWAVES = NT / 64;
     constexpr bool DGRAD = MODE == RING_DGRAD;
-    // Chunk j of tile row r sits at slot j ^ ((r >> SWZ) % CH).  With 32-row MFMA operands and 128-byte rows, two
-    // rows share 256 bytes of LDS and rows r and r+8 of an operand read would otherwise land on the same banks
+    // Chunk j of tile row r sits at slot j ^ ((r >> SWZ) % CH).  With 32-row MFMA operands and rows of 128 (64) bytes,
+    // two (four) rows share 256 bytes of LDS and rows r and r+8 (r+4) of an operand read would otherwise land on the same banks
     // (the counters showed every second LDS cycle of the data gradient as a bank conflict); the 16-row tilings
     // measure conflict-free as they are.
-    constexpr int SWZ = (MF == 32 && BK == 32) ? 1 : 0;
+    constexpr int SWZ = MF != 32 ? 0 : BK == 16 ? 2 : BK == 32 ? 1 : 0;  // log2 of the tile rows per 256 bytes
     // Copies are wave-wide: 64 lanes x 16 bytes = 1 KiB.  NAW / NBW of them make an A / B tile; every
     // wave issues the same number (NA + NB) per step so that all waves count outstanding copies alike;
     // where the tile does not divide evenly the surplus copies repeat an earlier one (same bytes twice).
