@@ -91,8 +91,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 pix_valid |= in ? (1u << (4 * r + s)) : 0u;
             }
     }
-    // where this thread's outputs go in a stage: row pr, 16-byte half (pc/4) swizzled by row bit 2
-    const int a_wr_off = pr * FBK + (((pc >> 2) ^ ((pr >> 2) & 1)) << 2) + (pc & 3);
+    // where this thread's outputs go in a stage: row pr, 16-byte half (pc/4) swizzled by row bit 3 (rows r and r+8 of an operand read share banks otherwise)
+    const int a_wr_off = pr * FBK + (((pc >> 2) ^ ((pr >> 3) & 1)) << 2) + (pc & 3);
 
     // ---- weight copies: 16-byte slot s = q*256 + tid of the chunk's [16][8][64] block ----------
     unsigned b_voff[FB_COPIES];
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const unsigned wave_lds = __builtin_amdgcn_readfirstlane(wave) * 1024u;
 
     // ---- consumer offsets (floats within a stage) -----------------------------------------------
-    const int a_rd_off = (wm0 + li) * FBK + ((lg ^ (((wm0 + li) >> 2) & 1)) << 2);
+    const int a_rd_off = (wm0 + li) * FBK + ((lg ^ (((wm0 + li) >> 3) & 1)) << 2);
     const int b_rd_off = FA_FLOATS + 4 * lg * FBN + wn0 + li;
 
     floatx16 P[16];
