@@ -91,36 +91,29 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(Cf
     // the group's first position: 0, or 8 for the second group
     const unsigned short *const a_first = TI16 + m0 * C + group * NPOS * a_pos_stride;
     const unsigned short *const b_first = Wt16 + static_cast<size_t>(n0) * C + group * NPOS * b_pos_stride;
-    const unsigned short *a_pos = a_first, *b_pos = b_first;
-    const unsigned short *a_next = a_pos, *b_next = b_pos;
-    int kc_next = 0, pos_next = 0;
-    unsigned slot_next = 0;
-    // Every thread issues exactly Cfg::COPIES copies per call; past the last step the walk wraps to
-    // the group's first position again (copied, never read).
+    // The walk over the (position, channel chunk) steps, branch-free: a step advances both pointers by BK
+    // channels, or by what takes them from a position's last chunk to the next position's first; after the
+    // group's last step they return to its first position (the surplus copies are never read).
+    const unsigned short *a_next = a_first, *b_next = b_first;
+    const size_t a_jump = a_pos_stride - static_cast<size_t>(nkc - 1) * BK, b_jump = b_pos_stride - static_cast<size_t>(nkc - 1) * BK;
+    int kc_left = nkc, steps_left = NPOS * nkc;
+    unsigned dst_next = smem_base;
+    // Every thread issues exactly Cfg::COPIES copies per call.
     auto issue = [&]() __attribute__((always_inline)) {
-        const unsigned dst = smem_base + slot_next * Cfg::STAGE_BYTES;
 #pragma unroll
-        for (int q = 0; q < PW; ++q) async_copy16(reinterpret_cast<const float *>(a_next), a_voff[q], dst + t_lds[q]);
+        for (int q = 0; q < PW; ++q) async_copy16(reinterpret_cast<const float *>(a_next), a_voff[q], dst_next + t_lds[q]);
 #pragma unroll
         for (int q = 0; q < PW; ++q)
-            async_copy16(reinterpret_cast<const float *>(b_next), b_voff[q], dst + Cfg::TILE_BYTES + t_lds[q]);
-        if (++kc_next == nkc) {
-            kc_next = 0;
-            if (++pos_next == NPOS) {
-                pos_next = 0;
-                a_pos = a_first;
-                b_pos = b_first;
-            } else {
-                a_pos += a_pos_stride;
-                b_pos += b_pos_stride;
-            }
-            a_next = a_pos;
-            b_next = b_pos;
-        } else {
-            a_next += BK;
-            b_next += BK;
+            async_copy16(reinterpret_cast<const float *>(b_next), b_voff[q], dst_next + Cfg::TILE_BYTES + t_lds[q]);
+        const bool last_chunk = --kc_left == 0;
+        kc_left = last_chunk ? nkc : kc_left;
+        a_next += last_chunk ? a_jump : static_cast<size_t>(BK);
+        b_next += last_chunk ? b_jump : static_cast<size_t>(BK);
+        if (--steps_left == 0) {
+            a_next = a_first;
+            b_next = b_first;
         }
-        slot_next = slot_next + 1 == NSTAGE ? 0 : slot_next + 1;
+        dst_next = dst_next + Cfg::STAGE_BYTES == smem_base + Cfg::LDS_BYTES ? smem_base : dst_next + Cfg::STAGE_BYTES;
     };
 
     floatx16 Y[4][1][1];
