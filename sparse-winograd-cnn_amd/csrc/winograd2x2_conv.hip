@@ -78,6 +78,8 @@ int conv_entry(const float *Input, const float *Weight, float *Output, int C, in
     if (!BF16) pick = choose_tiling(Input, Weight, M, C, K, true, true);
     note_conv_kernel(tiling_name(pick.tiling));
     switch (pick.tiling) {
+        case TILING_WIDE48:
+            return launch_wide48(Input, Weight, Output, M, C, K, nW, pick.wide, ep.scale, ep.shift, ep.residual, ep.residual_relu, s);
         case TILING_TALL16:
             return launch_async<Tall, 2, false>(Input, Weight, Output, M, C, K, nH, nW, pick.rows_per_wg, ep, s);
         case TILING_SHORT16:

@@ -39,6 +39,72 @@ inline size_t device_l2_bytes()
     return static_cast<size_t>(l2[dev]);
 }
 
+// How the wide48 kernel (winograd2x2_conv_wide_kernel.h) would cover M rows x N columns: `groups` row groups of
+// rows_per_wg <= 48 rows cover main_rows; with `extra` the rows beyond are dealt out as 16x16 tiles, one per
+// workgroup.  units: MFMA work of a wave per pass over the chip, in 16x16 tiles.
+struct WidePlan {
+    bool ok = false;
+    bool extra = false;
+    size_t groups = 0, rows_per_wg = 0, main_rows = 0, wgs = 0;
+    double units = 0;
+};
+
+// The kernel takes C in pairs of 32-channel steps, whole 128-column groups, 16-byte granules, 32-bit byte offsets
+// into the activations of one position and 31-bit ones into the output.
+inline bool wide48_eligible(const void *A, const void *B, size_t M, int R, int N)
+{
+    return R % 64 == 0 && N % 128 == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0 &&
+           M >= 48 && M * static_cast<size_t>(R) * 4 < (1ull << 32) && M * 16 * static_cast<size_t>(N) < (1ull << 31) &&
+           static_cast<size_t>(R) * N * 16 * 4 < (1ull << 40);
+}
+
+// Either full 48-row groups in whole passes over the chip with the rest as extra tiles (6.25 units per pass), or
+// the rows levelled over as many groups as fill whole passes (6 units), whichever makes fewer units in total.
+inline WidePlan plan_wide48(size_t M, int N, size_t cus)
+{
+    WidePlan best;
+    const size_t tiles_n = static_cast<size_t>(N) / 128;
+    if (tiles_n == 0 || M < 48) return best;
+    auto passes_of = [&](size_t wgs) { return static_cast<double>((wgs + cus - 1) / cus); };
+    {   // levelled
+        const size_t gmin = (M + 47) / 48;
+        const size_t wgs = (gmin * tiles_n + cus - 1) / cus * cus;
+        size_t groups = wgs / tiles_n > gmin ? wgs / tiles_n : gmin;
+        const size_t rows = (M + groups - 1) / groups;
+        groups = (M + rows - 1) / rows;
+        best.ok = true;
+        best.extra = false;
+        best.groups = groups;
+        best.rows_per_wg = rows;
+        best.main_rows = M;
+        best.wgs = groups * tiles_n;
+        best.units = passes_of(best.wgs) * 6.0;
+    }
+    {   // full groups plus extra tiles
+        const size_t gfull = M / 48;
+        size_t groups = gfull * tiles_n / cus * cus / tiles_n;
+        if (groups == 0) groups = gfull;
+        const size_t main_rows = groups * 48;
+        const size_t left_tiles = (M - main_rows + 15) / 16;
+        if (left_tiles > 0 && left_tiles * 8 <= groups) {
+            const double units = passes_of(groups * tiles_n) * 6.25;
+            if (units < best.units) {
+                best.extra = true;
+                best.groups = groups;
+                best.rows_per_wg = 48;
+                best.main_rows = main_rows;
+                best.wgs = groups * tiles_n;
+                best.units = units;
+            }
+        }
+    }
+    return best;
+}
+
+// Defined in winograd2x2_conv_wide.hip.
+int launch_wide48(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nW, const WidePlan &plan,
+                  const float *scale, const float *shift, const float *residual, int residual_relu, hipStream_t stream);
+
 namespace {
 
 // 32x32 MFMAs, wave tile 32x32: the fewest LDS reads per MFMA; its results are bit-identical to
@@ -50,7 +116,7 @@ using Tile16 = ConvCfg<64, 64, 16, 2, 2>;
 using Tall = ConvCfg<112, 64, 32, 1, 4, 2, 16>;
 using Short = ConvCfg<32, 64, 64, 1, 4, 3, 16>;
 
-enum Tiling { TILING_SYNC = 0, TILING_RING32, TILING_RING16, TILING_TALL16, TILING_SHORT16 };
+enum Tiling { TILING_SYNC = 0, TILING_RING32, TILING_RING16, TILING_TALL16, TILING_SHORT16, TILING_WIDE48 };
 inline const char *tiling_name(Tiling t)
 {
     switch (t) {
@@ -58,6 +124,7 @@ inline const char *tiling_name(Tiling t)
         case TILING_RING16: return "ring16";
         case TILING_TALL16: return "tall16";
         case TILING_SHORT16: return "short16";
+        case TILING_WIDE48: return "wide48";
         default: return "sync";
     }
 }
@@ -97,6 +164,7 @@ bool ring_eligible(const void *A, const void *B, int R, int N, bool forward)
 struct TilingChoice {
     Tiling tiling;
     size_t rows_per_wg;
+    WidePlan wide = WidePlan();  // TILING_WIDE48 only
 };
 
 // The tiling of a call with M rows, reduction length R and N output columns.  `ring16_ok`: the caller has a
@@ -118,8 +186,12 @@ inline TilingChoice choose_tiling(const void *A, const void *B, size_t M, int R,
     // tall16 levels its row groups over the CUs; short16 does better with full 32-row groups (two whole MFMA
     // tiles) even where that leaves some CUs with one workgroup more (conv4a: 69 vs 73 us).
     const size_t rows_tall = balanced_rows<Tall>(M, tiles_n, cus), rows_short = Short::BM;
+    // wide48 (forward only): 48-row x 128-column workgroups, left-over rows dealt out as extra tiles.
+    const bool ok_wide = forward && wide48_eligible(A, B, M, R, N);
+    const WidePlan wide = ok_wide ? plan_wide48(M, N, cus) : WidePlan();
     if (const char *f = forced_conv_tiling()) {
         const std::string_view want(f);
+        if (want == "wide48" && wide.ok) return {TILING_WIDE48, wide.rows_per_wg, wide};
         if (want == "ring32" && ok32) return {TILING_RING32, Tile32::BM};
         if (want == "ring16" && ok16) return {TILING_RING16, Tile16::BM};
         if (want == "tall16" && ok_tall) return {TILING_TALL16, rows_tall};
@@ -133,6 +205,9 @@ inline TilingChoice choose_tiling(const void *A, const void *B, size_t M, int R,
     const double cost32 = ok32 ? passes((M + 63) / 64 * tiles_n, cus) * 4.0 : 1e30;
     const double cost_tall = ok_tall ? passes(wgs_tall, cus) * 7.0 * w_tall : 1e30;
     const double cost_short = ok_short ? passes(wgs_short, cus) * 2.0 * w_short : 1e30;
+    // wide48: a unit of its work measured 9 % more than ring32's with one workgroup per CU, 1 % more with two.
+    const double cost_wide = wide.ok ? wide.units * (wide.wgs > cus ? 1.01 : 1.09) : 1e30;
+    if (wide.ok && cost_wide < cost32 && cost_wide < cost_tall && cost_wide < cost_short) return {TILING_WIDE48, wide.rows_per_wg, wide};
     if (ok_tall && cost_tall < cost32 && cost_tall <= cost_short) return {TILING_TALL16, rows_tall};
     if (ok_short && cost_short < cost32) return {TILING_SHORT16, rows_short};
     if (ok32) return {TILING_RING32, Tile32::BM};

@@ -138,11 +138,11 @@ def test_conv_shapes_reach_every_kernel(dev):
     import swc_hip
     _, conv = ops()
     seen = set()
-    for shape in CONV_SHAPES:
+    for shape in CONV_SHAPES + [(64, 14, 14, 128, 128)]:   # the last one: benchmark config 3, checked in full below
         B, nH, nW, C, K = shape
         conv(torch.zeros((16, B, nH, nW, C), device=dev), torch.zeros((16, C, K), device=dev))
         seen.add(swc_hip.lib().swc_winograd2x2_conv_last_kernel().decode())
-    assert seen == {"sync", "ring32", "ring16", "tall16", "short16"}, seen
+    assert seen == {"sync", "ring32", "ring16", "tall16", "short16", "wide48"}, seen
 
 
 @pytest.mark.parametrize("tiling", ["ring32", "ring16", "tall16", "short16", "sync"])
@@ -165,6 +165,54 @@ def test_conv_fp32_under_every_tiling(oracle, dev, shape, tiling):
         assert L.swc_winograd2x2_conv_force_tiling(None) == 0
     conv(gpu(ti, dev), gpu(w, dev))
     assert L.swc_winograd2x2_conv_last_kernel().decode() in ("ring32", "ring16", "tall16", "short16")
+
+
+# wide48 takes C % 64 == 0 and K % 128 == 0.  The shapes cover its two ways of dealing out the rows: levelled row
+# groups (down to one valid row per workgroup), and full 48-row groups with the rest as extra 16x16 tiles, whole and
+# ragged, with one and with two column groups.
+WIDE48_SHAPES = [
+    (8, 14, 14, 128, 128),   # levelled: 13 rows per workgroup
+    (3, 5, 7, 64, 128),      # levelled: M = 105 over 105 workgroups
+    (2, 20, 20, 64, 128),    # 16 full groups + 2 extra tiles
+    (2, 2, 197, 64, 128),    # 16 full groups + 20 rows: the second extra tile holds 4
+    (32, 1, 193, 64, 256),   # two column groups: 128 full groups + 2 extra row tiles
+    (8, 14, 14, 128, 256),   # two column groups, levelled
+]
+
+
+@pytest.mark.parametrize("shape", WIDE48_SHAPES)
+def test_conv_fp32_wide48(oracle, dev, shape):
+    """The wide48 tiling forced on shapes below the size at which the launcher picks it by itself.  Its output
+    transform is taken in another association than the reference's (sum/difference pairs, partial sums continued
+    by the matrix pipes), so besides the tolerance check the integer check pins every sign and the scatter exactly."""
+    import swc_hip
+    L = swc_hip.lib()
+    _, conv = ops()
+    B, nH, nW, C, K = shape
+    ti, w = conv_inputs(shape, 15, density=0.2)
+    rng = np.random.default_rng(16)
+    ti_int = rng.integers(-4, 5, size=(16, B, nH, nW, C)).astype(np.float32)
+    w_int = rng.integers(-4, 5, size=(16, C, K)).astype(np.float32)
+    scale = (0.5 + rng.random(K)).astype(np.float32) * rng.choice([-1, 1], K).astype(np.float32)
+    shift = rng.standard_normal(K).astype(np.float32)
+    res = rng.standard_normal((B, 2 * nH, 2 * nW, K)).astype(np.float32)
+    assert L.swc_winograd2x2_conv_force_tiling(b"wide48") == 0
+    try:
+        got = conv(gpu(ti, dev), gpu(w, dev))
+        assert L.swc_winograd2x2_conv_last_kernel().decode() == "wide48"
+        got_int = conv(gpu(ti_int, dev), gpu(w_int, dev)).cpu().numpy()
+        got_ep = conv(gpu(ti, dev), gpu(w, dev), scale=gpu(scale, dev), shift=gpu(shift, dev), residual=gpu(res, dev),
+                      residual_relu=True).cpu().numpy()
+        buf = gpu(res, dev)
+        conv(gpu(ti, dev), gpu(w, dev), out=buf, residual=buf)   # residual aliasing the output
+    finally:
+        assert L.swc_winograd2x2_conv_force_tiling(None) == 0
+    want = oracle.conv(ti, w, acc64=True)
+    assert rel_max(got.cpu().numpy(), want) <= TOL and rel_l1(got.cpu().numpy(), want) <= TOL
+    assert np.array_equal(got_int, oracle.conv(ti_int, w_int))
+    # the epilogue's own arithmetic is exact against the oracle's on the kernel's plain output
+    assert np.array_equal(got_ep, oracle.affine(got.cpu().numpy(), scale, shift) + np.maximum(res, 0))
+    assert np.array_equal(buf.cpu().numpy(), got.cpu().numpy() + res)
 
 
 @pytest.mark.parametrize("shape", [(3, 3, 3, 32, 32), (2, 4, 4, 5, 7), (2, 3, 5, 36, 100), (8, 9, 9, 128, 72),
