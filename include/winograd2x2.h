@@ -281,8 +281,15 @@ SWC_API int swc_winograd2x2_conv_grad(const float *TInput, const float *Weight, 
  * B*nH*nW*K <= 1 048 576; larger calls return SWC_ERR_TOO_LARGE and launch nothing).  Nothing is allocated or
  * freed, by this call or by anything it calls.  All calls on one GPU share that array: calls that may overlap on
  * one GPU (different streams or host threads) race on it and must be serialised by the caller.
+ * The first call on a device looks up the array's address there (hipGetDevice and hipGetSymbolAddress, under a
+ * mutex): a caller that captures HIP graphs makes one call on the device outside the capture first.
+ * The array is part of the library's code object, so every process that loads the library holds its 64 MiB on every
+ * GPU it uses, whether or not it calls this entry point; a build for forward-only deployments can shrink it with
+ * -DSWC_CONV_GRAD_STATIC_MAX_FLOATS=<n>.
  */
+#ifndef SWC_CONV_GRAD_STATIC_MAX_FLOATS
 #define SWC_CONV_GRAD_STATIC_MAX_FLOATS (16u << 20)
+#endif
 SWC_API int swc_winograd2x2_conv_grad_static(const float *TInput, const float *Weight, const float *Output_grad,
                                              float *TInput_grad, float *Weight_grad, int C, int B, int H, int W,
                                              int K, int pad_h, int pad_w, swc_stream_t stream);
@@ -313,6 +320,44 @@ SWC_API int swc_winograd2x2_imtrans_grad(const float *TransIm_grad, const float 
 SWC_API int swc_winograd2x2_imtrans_grad_relu_input(const float *TransIm_grad, const float *Input,
                                                     float *Input_grad, int C, int B, int H, int W,
                                                     int pad_h, int pad_w, swc_stream_t stream);
+
+/*
+ * Shape rule of Winograd2x2ConvGrad: TInput [16,B,nH,nW,C], Weight [16,C,K], Output_grad [B,H,W,K] with
+ * H = 2nH, W = 2nW -> the two results shaped like TInput and Weight, and the number of floats of the temporary
+ * the launcher needs (16*nH*nW*B*K), as Winograd2x2ConvGradCudaOp::Compute derives them
+ * (winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_grad_op.cc:44-67).  The reference checks nothing; this
+ * also requires that the three shapes agree.
+ */
+SWC_API int swc_winograd2x2_conv_grad_op_shape(int ti_rank, const int64_t *ti_dims, int w_rank, const int64_t *w_dims,
+                                       int g_rank, const int64_t *g_dims, int64_t ti_grad_dims[5],
+                                       int64_t w_grad_dims[3], int64_t *tmp_floats);
+
+/*
+ * Winograd2x2ConvGradCudaOp::Compute (winograd2x2_conv_grad_op.cc:36-78) with the two results and the temporary
+ * passed in (tmp_floats: how many floats tmp_data_buffer holds); launches with pad 1,1.
+ */
+SWC_API int swc_winograd2x2_conv_grad_op_compute(const float *tinput, int ti_rank, const int64_t *ti_dims,
+                                         const float *weight, int w_rank, const int64_t *w_dims,
+                                         const float *output_grad, int g_rank, const int64_t *g_dims,
+                                         float *tinput_grad, float *weight_grad, float *tmp_data_buffer,
+                                         int64_t tmp_floats, swc_stream_t stream);
+
+/*
+ * Shape rule of Winograd2x2ImTransGrad: Output_grad [16,B,nH,nW,C] -> [B,2nH,2nW,C]
+ * (winograd2x2_cublas/winograd2x2_imTrans/winograd2x2_imTrans_grad_op.cc:40-49).
+ */
+SWC_API int swc_winograd2x2_imtrans_grad_op_shape(int g_rank, const int64_t *g_dims, int64_t in_grad_dims[4]);
+
+/*
+ * Winograd2x2ImTransGradCudaOp::Compute (winograd2x2_imTrans_grad_op.cc:33-55) with the result passed in.
+ * ig_dims is [B,H,W,C] with H = 2nH as in the reference, or 2nH - 1 for a forward input of odd extent (likewise
+ * W).  relu_output / relu_input: at most one of them, the source of the fused ReLU's mask as in
+ * swc_winograd2x2_imtrans_grad / swc_winograd2x2_imtrans_grad_relu_input; both NULL: no ReLU, as in the reference.
+ */
+SWC_API int swc_winograd2x2_imtrans_grad_op_compute(const float *output_grad, int g_rank, const int64_t *g_dims,
+                                            const float *relu_output, const float *relu_input,
+                                            float *input_grad, int ig_rank, const int64_t *ig_dims,
+                                            swc_stream_t stream);
 
 #ifdef __cplusplus
 } /* extern "C" */

@@ -328,8 +328,13 @@ __global__ __launch_bounds__(256) void gemm16_plain_kernel(const float *__restri
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const int row = ty + 8 * k;  // tile row: p for A, r for B
-            const int pa = p0 + row, ra = r0 + tx;
-            As[row][tx] = pa < P && ra < Rn ? a[pa * a_p + ra * a_r] : 0.f;
+            if (a_p == 1) {  // p is A's fast axis (dW: A = TI^T): the 32 lanes walk p so that a load is one 128-byte line
+                const int pa = p0 + tx, ra = r0 + row;
+                As[tx][row] = pa < P && ra < Rn ? a[pa + ra * a_r] : 0.f;
+            } else {
+                const int pa = p0 + row, ra = r0 + tx;
+                As[row][tx] = pa < P && ra < Rn ? a[pa * a_p + ra * a_r] : 0.f;
+            }
             const int rb = r0 + row, qb = q0 + tx;
             Bs[row][tx] = rb < Rn && qb < Q ? b[rb * b_r + qb * b_q] : 0.f;
         }
@@ -442,7 +447,10 @@ int conv_grad_impl(const float *TInput, const float *Weight, const float *Output
     if (C <= 0 || B <= 0 || H <= 0 || W <= 0 || K <= 0 || (H & 1) || (W & 1)) return SWC_ERR_BAD_DIMS;  // H = 2nH, W = 2nW
     if (pad_h != 1 || pad_w != 1) return SWC_ERR_BAD_PAD;
     const int nH = H / 2, nW = W / 2;
-    const size_t M = static_cast<size_t>(B) * nH * nW;
+    // each factor is below 2^31, so B*nH fits 64 bits; the bound on it keeps the next product from wrapping
+    const size_t bh = static_cast<size_t>(B) * nH;
+    if (bh >= (1ull << 31)) return SWC_ERR_BAD_DIMS;
+    const size_t M = bh * nW;
     if (M >= (1ull << 31) || M * K >= (1ull << 32) || M * C >= (1ull << 40)) return SWC_ERR_BAD_DIMS;
 
     const bool vec = (K % 4 == 0) && aligned16(Output_grad) && aligned16(dP);
@@ -526,8 +534,12 @@ extern "C" int swc_winograd2x2_conv_grad_static(const float *TInput, const float
                                                 int pad_h, int pad_w, swc_stream_t stream)
 {
     if (C <= 0 || B <= 0 || H <= 0 || W <= 0 || K <= 0 || (H & 1) || (W & 1)) return SWC_ERR_BAD_DIMS;
-    const size_t need = static_cast<size_t>(16) * B * (H / 2) * (W / 2) * K;  // floats of dP
-    if (need > swc::kStaticScratchFloats) return SWC_ERR_TOO_LARGE;
+    // dP holds 16*M*K floats, M = B*(H/2)*(W/2).  The products are bounded one factor at a time: a product of
+    // four ints taken at once could wrap to a small value and slip past the limit.
+    const size_t bh = static_cast<size_t>(B) * (H / 2);
+    if (bh > swc::kStaticScratchFloats) return SWC_ERR_TOO_LARGE;
+    const size_t M = bh * (W / 2);
+    if (M > swc::kStaticScratchFloats || M * K > swc::kStaticScratchFloats / 16) return SWC_ERR_TOO_LARGE;
     int st = SWC_OK;
     float *dP = swc::static_scratch(&st);
     if (dP == nullptr) return st;

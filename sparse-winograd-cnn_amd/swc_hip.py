@@ -29,6 +29,8 @@ C_SYMBOLS = (
     "swc_winograd2x2_relu_conv_bf16",
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
+    "swc_winograd2x2_conv_grad_op_shape", "swc_winograd2x2_conv_grad_op_compute",
+    "swc_winograd2x2_imtrans_grad_op_shape", "swc_winograd2x2_imtrans_grad_op_compute",
     "swc_winograd2x2_conv_grad", "swc_winograd2x2_imtrans_grad", "swc_winograd2x2_imtrans_grad_relu_input",
     "swc_winograd2x2_relu_conv", "swc_winograd2x2_pointwise_conv",
 )
@@ -109,6 +111,15 @@ def lib():
         L.swc_winograd2x2_conv_op_compute.argtypes = [fp, i32, i64p, fp, i32, i64p, fp, i32, i64p, i32, vp]
         L.swc_winograd2x2_relu_conv.restype = i32
         L.swc_winograd2x2_relu_conv.argtypes = [fp] * 3 + [i32] * 8 + [vp]
+        L.swc_winograd2x2_conv_grad_op_shape.restype = i32
+        L.swc_winograd2x2_conv_grad_op_shape.argtypes = [i32, i64p, i32, i64p, i32, i64p, i64p, i64p, i64p]
+        L.swc_winograd2x2_conv_grad_op_compute.restype = i32
+        L.swc_winograd2x2_conv_grad_op_compute.argtypes = [fp, i32, i64p, fp, i32, i64p, fp, i32, i64p, fp, fp, fp,
+                                                           ctypes.c_int64, vp]
+        L.swc_winograd2x2_imtrans_grad_op_shape.restype = i32
+        L.swc_winograd2x2_imtrans_grad_op_shape.argtypes = [i32, i64p, i64p]
+        L.swc_winograd2x2_imtrans_grad_op_compute.restype = i32
+        L.swc_winograd2x2_imtrans_grad_op_compute.argtypes = [fp, i32, i64p, fp, fp, fp, i32, i64p, vp]
         L.swc_winograd2x2_conv_grad.restype = i32
         L.swc_winograd2x2_conv_grad.argtypes = [fp] * 7 + [i32] * 7 + [vp]
         L.swc_winograd2x2_imtrans_grad.restype = i32

@@ -5,6 +5,7 @@ Mirrors winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv.py of the reference
 (:19-29), ``winograd2x2_conv_grad(i1, i2, grad)`` (:16-17), and the gradient registration
 (:31-36) as a torch.autograd.Function.
 """
+import ctypes
 import os
 import sys
 
@@ -132,23 +133,30 @@ def _forward_bf16_stored(I, W, out, scale, shift, residual, residual_relu=False)
     return out
 
 
+def winograd2x2_conv_grad_shape(i_shape, w_shape, g_shape):
+    """(I.shape, W.shape, grad.shape) -> (dI shape, dW shape, floats of the launcher's temporary), by the host op
+    wrapper (swc_winograd2x2_conv_grad_op_shape; winograd2x2_conv_grad_op.cc:44-67)."""
+    ti_g, w_g, tmp = swc_hip.dims([0] * 5), swc_hip.dims([0] * 3), ctypes.c_int64(0)
+    swc_hip.check(swc_hip.lib().swc_winograd2x2_conv_grad_op_shape(
+        len(i_shape), swc_hip.dims(i_shape), len(w_shape), swc_hip.dims(w_shape), len(g_shape), swc_hip.dims(g_shape),
+        ti_g, w_g, ctypes.byref(tmp)), "winograd2x2_conv_grad")
+    return tuple(ti_g), tuple(w_g), int(tmp.value)
+
+
 def winograd2x2_conv_grad(i1, i2, grad):
     """(I [16,B,nH,nW,C], W [16,C,K], grad [B,2nH,2nW,K]) -> (dI, dW), as the reference's
     winograd2x2_conv_grad (winograd2x2_conv.py:16-17).  fp32 throughout."""
     I = swc_hip.require_cuda_f32(i1, "i1", 5)
     W = swc_hip.require_cuda_f32(i2, "i2", 3)
     grad = swc_hip.require_cuda_f32(grad, "grad", 4)
-    want = winograd2x2_conv_shape(I.shape, W.shape)
-    if tuple(grad.shape) != want:
-        raise ValueError("grad must have shape %s, got %s" % (want, tuple(grad.shape)))
-    _, B, nH, nW, C = I.shape
-    K = W.shape[2]
-    dI, dW = torch.empty_like(I), torch.empty_like(W)
-    tmp = torch.empty(16 * B * nH * nW * K, dtype=torch.float32, device=I.device)  # as winograd2x2_conv_grad_op.cc:69-71
+    di_shape, dw_shape, tmp_floats = winograd2x2_conv_grad_shape(I.shape, W.shape, grad.shape)
+    dI = torch.empty(di_shape, dtype=torch.float32, device=I.device)
+    dW = torch.empty(dw_shape, dtype=torch.float32, device=I.device)
+    tmp = torch.empty(tmp_floats, dtype=torch.float32, device=I.device)  # as winograd2x2_conv_grad_op.cc:66-67
     with swc_hip.on_device(I.device) as stream:
-        st = swc_hip.lib().swc_winograd2x2_conv_grad(
-            I.data_ptr(), W.data_ptr(), grad.data_ptr(), dI.data_ptr(), dW.data_ptr(), tmp.data_ptr(), None,
-            C, B, 2 * nH, 2 * nW, K, 1, 1, stream)
+        st = swc_hip.lib().swc_winograd2x2_conv_grad_op_compute(
+            I.data_ptr(), 5, swc_hip.dims(I.shape), W.data_ptr(), 3, swc_hip.dims(W.shape), grad.data_ptr(), 4,
+            swc_hip.dims(grad.shape), dI.data_ptr(), dW.data_ptr(), tmp.data_ptr(), tmp_floats, stream)
     swc_hip.check(st, "winograd2x2_conv_grad")
     return dI, dW
 

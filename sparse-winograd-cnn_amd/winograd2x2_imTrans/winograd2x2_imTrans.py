@@ -108,12 +108,10 @@ def winograd2x2_imTrans_grad(grad, H=None, W=None, relu_output=None, relu_input=
         mask_ptr = relu_output.data_ptr()
     out = torch.empty((B, H, W, C), dtype=torch.float32, device=grad.device)
     with swc_hip.on_device(grad.device) as stream:
-        if relu_input is not None:
-            st = swc_hip.lib().swc_winograd2x2_imtrans_grad_relu_input(grad.data_ptr(), relu_input.data_ptr(),
-                                                                       out.data_ptr(), C, B, H, W, 1, 1, stream)
-        else:
-            st = swc_hip.lib().swc_winograd2x2_imtrans_grad(grad.data_ptr(), mask_ptr, out.data_ptr(), C, B, H, W, 1, 1,
-                                                            stream)
+        # the host op wrapper (winograd2x2_imTrans_grad_op.cc:33-55) checks the shapes against each other again
+        st = swc_hip.lib().swc_winograd2x2_imtrans_grad_op_compute(
+            grad.data_ptr(), 5, swc_hip.dims(grad.shape), mask_ptr, None if relu_input is None else relu_input.data_ptr(),
+            out.data_ptr(), 4, swc_hip.dims(out.shape), stream)
     swc_hip.check(st, "winograd2x2_imTrans_grad")
     return out
 

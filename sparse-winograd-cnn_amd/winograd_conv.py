@@ -49,9 +49,12 @@ class WinogradConv(torch.nn.Module):
         self._bf16 = None
 
     def refresh(self):
-        """Drop the cached W*mask and its bf16 copy.  Not needed after in-place updates of W or mask
-        (optimizer steps, ``load_state_dict``): the caches are keyed on the tensors' version counters
-        and storage, so those are noticed by themselves."""
+        """Drop the cached W*mask and its bf16 copy.  Not needed after in-place updates of W or mask made on
+        the tensors themselves or on ``detach()``ed views of them (optimizer steps, ``load_state_dict``,
+        ``with torch.no_grad(): W.mul_(m)``): the caches are keyed on the tensors' version counters and storage,
+        so those are noticed by themselves.  Needed after a write through ``.data`` (``layer.W.data.mul_(m)``,
+        ``layer.W.data.copy_(w)``): a ``.data`` view carries a version counter of its own, so such a write leaves
+        no trace on W."""
         self._masked = None
         self._bf16 = None
 
@@ -70,13 +73,14 @@ class WinogradConv(torch.nn.Module):
         return cached[1]
 
     def masked_weight(self):
-        """W*mask without autograd history, recomputed only when W or mask changed since the last call."""
+        """W*mask without autograd history, recomputed only when W or mask changed since the last call (a write
+        through ``.data`` is not such a change: see refresh())."""
         if self.mask is None:
-            return self.W.data
+            return self.W.detach()   # shares W's version counter: a write to what is handed out is noticed
         key = self._weight_key()
         cached = self._masked
         if cached is None or cached[0] != key:
-            cached = (key, (self.W.data * self.mask).contiguous())
+            cached = (key, (self.W.detach() * self.mask).contiguous())
             self._masked = cached
         return cached[1]
 

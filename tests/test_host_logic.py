@@ -173,6 +173,25 @@ def test_masked_weight_cache_follows_weight_updates():
     with torch.no_grad():
         plain.W.mul_(2.0)
     assert plain._weight_key() != k1
+    k2 = plain._weight_key()
+    plain.masked_weight().mul_(0.5)                            # a write to what the layer hands out is noticed too
+    assert plain._weight_key() != k2
+
+
+def test_writes_through_dot_data_need_refresh():
+    """A `.data` view has a version counter of its own: W*mask and the bf16 copy keep their old values after
+    `layer.W.data.mul_()` until refresh() is called, as the docstrings of refresh() and masked_weight() say."""
+    from winograd_conv import WinogradConv
+    m = torch.ones(16, 4, 6)
+    m[:, :, ::2] = 0
+    layer = WinogradConv(4, 6, mask=m.numpy(), W_init=lambda w: w.fill_(2.0))
+    assert torch.equal(layer.masked_weight(), m * 2.0)
+    layer.W.data.mul_(3.0)
+    assert torch.equal(layer.masked_weight(), m * 2.0)         # stale: nothing recorded the write
+    layer.refresh()
+    assert torch.equal(layer.masked_weight(), m * 6.0)
+    layer.W.detach().mul_(0.5)                                 # the detach() view shares W's counter: noticed
+    assert torch.equal(layer.masked_weight(), m * 3.0)
 
 
 def test_weight_preparation_matches_oracle(oracle):
@@ -184,3 +203,54 @@ def test_weight_preparation_matches_oracle(oracle):
     w1, w2 = w.copy(), w.copy()
     assert np.array_equal(gen_prune_mask(w1, 0.2), oracle.gen_prune_mask(w2, 0.2))
     assert np.array_equal(w1, w2) and int((w1 != 0).sum()) == int(w.size * 0.2)
+
+
+def test_gradient_op_shape_rules():
+    """The host wrappers of the two gradient ops: winograd2x2_conv_grad_op.cc:44-67 (results shaped like the
+    inputs, temporary of 16*nH*nW*B*K floats) and winograd2x2_imTrans_grad_op.cc:40-49 (H = 2nH)."""
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv_grad_shape
+    L = swc_hip.lib()
+    assert winograd2x2_conv_grad_shape((16, 64, 14, 14, 128), (16, 128, 128), (64, 28, 28, 128)) == (
+        (16, 64, 14, 14, 128), (16, 128, 128), 16 * 14 * 14 * 64 * 128)
+    assert winograd2x2_conv_grad_shape((16, 2, 4, 4, 5), (16, 5, 7), (2, 8, 8, 7)) == ((16, 2, 4, 4, 5), (16, 5, 7), 16 * 32 * 7)
+    ti, w, g = swc_hip.dims((16, 2, 4, 4, 5)), swc_hip.dims((16, 5, 7)), swc_hip.dims((2, 8, 8, 7))
+    o5, o3, tmp = swc_hip.dims([0] * 5), swc_hip.dims([0] * 3), ctypes.c_int64(0)
+    ok = lambda *a: L.swc_winograd2x2_conv_grad_op_shape(*a, o5, o3, ctypes.byref(tmp))
+    assert ok(5, ti, 3, w, 4, g) == 0
+    assert ok(4, ti, 3, w, 4, g) == swc_hip.SWC_ERR_BAD_RANK
+    assert ok(5, ti, 3, w, 3, g) == swc_hip.SWC_ERR_BAD_RANK
+    assert ok(5, ti, 3, w, 4, swc_hip.dims((2, 7, 8, 7))) == swc_hip.SWC_ERR_BAD_DIMS      # the output is never cropped: H = 2nH
+    assert ok(5, ti, 3, w, 4, swc_hip.dims((3, 8, 8, 7))) == swc_hip.SWC_ERR_BAD_DIMS      # B disagrees
+    assert ok(5, ti, 3, swc_hip.dims((16, 5, 8)), 4, g) == swc_hip.SWC_ERR_BAD_DIMS        # K disagrees
+    assert ok(5, ti, 3, swc_hip.dims((16, 6, 7)), 4, g) == swc_hip.SWC_ERR_BAD_DIMS        # C disagrees
+    assert ok(5, None, 3, w, 4, g) == swc_hip.SWC_ERR_NULL_POINTER
+    # compute: a temporary that is too small is refused before anything is launched
+    p = ctypes.c_void_p(4096)
+    assert L.swc_winograd2x2_conv_grad_op_compute(p, 5, ti, p, 3, w, p, 4, g, p, p, p, 16 * 32 * 7 - 1, None) == swc_hip.SWC_ERR_BAD_DIMS
+
+    o4 = swc_hip.dims([0] * 4)
+    assert L.swc_winograd2x2_imtrans_grad_op_shape(5, swc_hip.dims((16, 64, 4, 4, 512)), o4) == 0
+    assert tuple(o4) == (64, 8, 8, 512)                                                        # 2nH, not the forward 7
+    assert L.swc_winograd2x2_imtrans_grad_op_shape(4, swc_hip.dims((16, 64, 4, 4)), o4) == swc_hip.SWC_ERR_BAD_RANK
+    assert L.swc_winograd2x2_imtrans_grad_op_shape(5, swc_hip.dims((15, 64, 4, 4, 512)), o4) == swc_hip.SWC_ERR_BAD_RANK
+    assert L.swc_winograd2x2_imtrans_grad_op_shape(5, swc_hip.dims((16, 64, 0, 4, 512)), o4) == swc_hip.SWC_ERR_BAD_DIMS
+    g5 = swc_hip.dims((16, 2, 4, 4, 8))
+    bad = lambda ig, ro=None, ri=None: L.swc_winograd2x2_imtrans_grad_op_compute(p, 5, g5, ro, ri, p, 4, swc_hip.dims(ig), None)
+    assert bad((2, 6, 8, 8)) == swc_hip.SWC_ERR_BAD_DIMS       # 6 does not tile into 4
+    assert bad((2, 9, 8, 8)) == swc_hip.SWC_ERR_BAD_DIMS
+    assert bad((2, 8, 8, 9)) == swc_hip.SWC_ERR_BAD_DIMS
+    assert bad((2, 8, 8, 8), p, p) == swc_hip.SWC_ERR_BAD_DIMS  # two sources for the mask
+
+
+def test_static_entry_bounds_its_size_one_factor_at_a_time():
+    """16*B*(H/2)*(W/2)*K taken as one product of ints can wrap to a small number; the entry point must refuse such
+    dimensions before it touches the GPU (the pointers here are never dereferenced)."""
+    L = swc_hip.lib()
+    p = ctypes.c_void_p(4096)
+    big = 2 ** 31 - 2
+    for dims in ((1, big, big, big, big), (1, 2 ** 16, 2 ** 17, 2 ** 17, 2 ** 16), (1, 2 ** 30, 4, 4, 2 ** 30),
+                 (1, 2, 2, 2, 2 ** 21)):
+        C, B, H, W, K = dims
+        assert L.swc_winograd2x2_conv_grad_static(p, p, p, p, p, C, B, H, W, K, 1, 1, None) == swc_hip.SWC_ERR_TOO_LARGE, dims
+        if dims[1] > 2:   # and the allocating entry refuses what no buffer could hold (the last case is valid there)
+            assert L.swc_winograd2x2_conv_grad(p, p, p, p, p, p, None, C, B, H, W, K, 1, 1, None) == swc_hip.SWC_ERR_BAD_DIMS, dims

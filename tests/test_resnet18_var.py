@@ -180,5 +180,11 @@ def test_layers_at_batch_128(oracle, hw, C, K, precision):
     if precision == "fp32":
         assert kernel != "sync", kernel   # every model shape runs on one of the copy-ring tilings
     if stored:
-        # more tiles than CUs at every layer; weights of 4 MiB and more (an L2) take the deeper ring
-        assert kernel == ("stored-ring4" if 16 * C * K * 2 >= (4 << 20) else "stored-ring3"), kernel
+        # The launcher reads the CU count and the L2 size from the device; so does the expectation.  More 64x64
+        # tiles than CUs at every layer of an MI355X; weights that fill an L2 (4 MiB there) take the deeper ring.
+        props = torch.cuda.get_device_properties(dev)
+        tiles = -(-N * ((hw + 1) // 2) ** 2 // 64) * -(-K // 64)
+        if tiles <= props.multi_processor_count:
+            assert kernel == "stored-split", kernel
+        else:
+            assert kernel == ("stored-ring4" if 16 * C * K * 2 >= props.L2_cache_size else "stored-ring3"), kernel

@@ -39,7 +39,8 @@ def test_static_scratch_entry_point_matches_the_allocating_one():
     dev = torch.device("cuda:0")
     rng = np.random.default_rng(77)
     # two calls in a row, the second with a smaller input: it must not see the first call's leftovers
-    for shape in ((8, 7, 7, 128, 64), (2, 3, 5, 36, 20)):
+    # the first one fills the array exactly: B*nH*nW*K = 1 048 576
+    for shape in ((16, 16, 16, 64, 256), (8, 7, 7, 128, 64), (2, 3, 5, 36, 20)):
         (dti_a, dw_a), (dti_s, dw_s) = _both(L, dev, rng, *shape)
         assert np.isfinite(dti_a).all() and np.isfinite(dw_a).all()
         # same kernels on the same inputs: bit for bit
@@ -57,3 +58,5 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit():
     assert st == swc_hip.SWC_ERR_TOO_LARGE
     assert b"scratch" in L.swc_strerror(st)
     assert L.swc_winograd2x2_conv_grad_static(p, p, p, p, p, 128, 64, 27, 28, 128, 1, 1, None) == swc_hip.SWC_ERR_BAD_DIMS
+    # one float more than fits
+    assert L.swc_winograd2x2_conv_grad_static(p, p, p, p, p, 64, 16, 32, 32, 257, 1, 1, None) == swc_hip.SWC_ERR_TOO_LARGE
