@@ -189,6 +189,25 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
     ep.residual = Residual;
     ep.residual_relu = residual_relu != 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // Layers of 128, 256 or 512 channels with enough 128-row x 64-column tiles for three quarters of the CUs: the
+    // tall tiles (twice the matrix work per byte through LDS, which bounds these layers: 14x14 at batch 128,
+    // 512 -> 512 77 us against 100, 28x28, 128 -> 128 27 against 35; with a residual to add 35 against 58).  With more
+    // tiles than CUs two workgroups share a CU and the rows are levelled over whole rounds of them.
+    if (bf16_tall_eligible(Input16, Weight16t, M, C, K)) {
+        const size_t tall_n = static_cast<size_t>(K) / 64, tall_m = (M + 127) / 128;
+        if (tall_m * tall_n * 4 >= 3 * cus) {
+            size_t tall_rows = 128;
+            if (tall_m * tall_n > cus) {
+                const size_t slots = 2 * cus, wgs = (tall_m * tall_n + slots - 1) / slots * slots;
+                const size_t groups = wgs / tall_n > tall_m ? wgs / tall_n : tall_m;
+                tall_rows = (M + groups - 1) / groups;
+                if (tall_rows > 128) tall_rows = 128;
+                if (tall_rows < 64) tall_rows = 64;
+            }
+            note_conv_kernel("stored-tall");
+            return launch_bf16_tall(Input16, Weight16t, Output, M, C, K, nW, tall_rows, Scale, Shift, Residual, residual_relu != 0, s);
+        }
+    }
     // A grid of full tiles that leaves every CU with one workgroup at most: the launch then lasts as long as one
     // workgroup's chain of steps, and splitting the 16 positions over two groups of waves halves the chain
     // (7x7x512 at batch 64: 30.7 us against 37.1; 14x14x256: 19.9 against 22.9).

@@ -101,6 +101,12 @@ inline WidePlan plan_wide48(size_t M, int N, size_t cus)
     return best;
 }
 
+// Defined in winograd2x2_conv_bf16_tall.hip: the bf16-stored convolution over 128-row x 64-column tiles.
+bool bf16_tall_eligible(const void *TI16, const void *Wt16, size_t M, int C, int K);
+int launch_bf16_tall(const unsigned short *TI16, const unsigned short *Wt16, float *Out, size_t M, int C, int K, int nW,
+                     size_t rows_per_wg, const float *scale, const float *shift, const float *residual, int residual_relu,
+                     hipStream_t stream);
+
 // Defined in winograd2x2_conv_wide.hip.
 int launch_wide48(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nW, const WidePlan &plan,
                   const float *scale, const float *shift, const float *residual, int residual_relu, hipStream_t stream);

@@ -97,6 +97,51 @@ def test_conv_over_bf16_operands(oracle, dev, shape):
         assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() in (b"stored-ring3", b"stored-ring4")
 
 
+@pytest.mark.parametrize("shape", [
+    (6, 16, 16, 128, 1024),   # 12 x 16 tiles of 128 rows x 64 columns
+    (3, 20, 25, 256, 1024),   # M = 1500: the last row group holds 92 rows
+    (2, 16, 24, 512, 2048),   # 512 channels: eight steps per position
+    (4, 25, 25, 128, 1024),   # more tiles than CUs: rows levelled over whole rounds (79 per workgroup on an MI355X)
+])
+def test_stored_tall_kernel(oracle, dev, shape):
+    """Layers of 128, 256 or 512 channels with enough tiles for the chip run `stored-tall` (128-row x 64-column
+    workgroups, the output transform in the sum/difference association): values against the oracle fed the same
+    bf16 operands, exactly on integers (every sign and the scatter), and the epilogue's arithmetic exactly."""
+    import swc_hip
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv, winograd2x2_weights_bf16
+    B, nH, nW, C, K = shape
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    if -(-B * nH * nW // 128) * (K // 64) * 4 < 3 * cus:
+        pytest.skip("this device has too many CUs for the shape to take the tall tiles")
+    rng = np.random.default_rng(67)
+    ti = np.maximum(rng.standard_normal((16, B, nH, nW, C)), 0).astype(np.float32)
+    w = (rng.standard_normal((16, C, K)) * 0.05).astype(np.float32)
+    ti16, w16 = oracle.round_bf16(ti), oracle.round_bf16(w)
+    ti_gpu, w_gpu = gpu(ti16, dev).to(torch.bfloat16), winograd2x2_weights_bf16(gpu(w, dev))
+    got = winograd2x2_conv(ti_gpu, w_gpu).cpu().numpy()
+    assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() == b"stored-tall"
+    want = oracle.conv(ti16, w16, acc64=True)
+    assert got.shape == want.shape
+    assert rel_max(got, want) <= TOL
+    # small integers: exact in bf16 and in every partial sum
+    ti_i = rng.integers(-3, 4, size=ti.shape).astype(np.float32)
+    w_i = rng.integers(-3, 4, size=w.shape).astype(np.float32)
+    got_i = winograd2x2_conv(gpu(ti_i, dev).to(torch.bfloat16), gpu(w_i, dev)).cpu().numpy()
+    assert np.array_equal(got_i, oracle.conv(ti_i, w_i))
+    # the epilogue
+    scale = (0.5 + rng.random(K)).astype(np.float32) * rng.choice([-1, 1], K).astype(np.float32)
+    shift = rng.standard_normal(K).astype(np.float32)
+    res = rng.standard_normal(want.shape).astype(np.float32)
+    got2 = winograd2x2_conv(ti_gpu, w_gpu, scale=gpu(scale, dev), shift=gpu(shift, dev), residual=gpu(res, dev)).cpu().numpy()
+    assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() == b"stored-tall"
+    assert np.array_equal(got2, oracle.affine(got, scale, shift) + res)
+    got3 = winograd2x2_conv(ti_gpu, w_gpu, residual=gpu(res, dev), residual_relu=True).cpu().numpy()
+    assert np.array_equal(got3, got + np.maximum(res, 0))
+    buf = gpu(res, dev)
+    winograd2x2_conv(ti_gpu, w_gpu, out=buf, residual=buf)      # residual aliasing the output
+    assert np.array_equal(buf.cpu().numpy(), got + res)
+
+
 def test_unsupported_channel_count_is_reported(dev):
     from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv
     import swc_hip

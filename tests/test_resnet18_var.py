@@ -183,8 +183,11 @@ def test_layers_at_batch_128(oracle, hw, C, K, precision):
         # The launcher reads the CU count and the L2 size from the device; so does the expectation.  More 64x64
         # tiles than CUs at every layer of an MI355X; weights that fill an L2 (4 MiB there) take the deeper ring.
         props = torch.cuda.get_device_properties(dev)
-        tiles = -(-N * ((hw + 1) // 2) ** 2 // 64) * -(-K // 64)
-        if tiles <= props.multi_processor_count:
+        M = N * ((hw + 1) // 2) ** 2
+        tiles = -(-M // 64) * -(-K // 64)
+        if C in (128, 256, 512) and K % 64 == 0 and -(-M // 128) * (K // 64) * 4 >= 3 * props.multi_processor_count:
+            assert kernel == "stored-tall", kernel      # enough 128-row x 64-column tiles to go round
+        elif tiles <= props.multi_processor_count:
             assert kernel == "stored-split", kernel
         else:
             assert kernel == ("stored-ring4" if 16 * C * K * 2 >= props.L2_cache_size else "stored-ring3"), kernel
