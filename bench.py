@@ -28,19 +28,20 @@ for _p in (ROOT, PKG):
 
 # Memory traffic per launch (bytes) behind the L2s, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
 # dispatch) and scaled by what the same counters read for a 128 MiB copy: FETCH_SIZE x 2.00, WRITE_SIZE x 1.00
-# (profiles/*_pmc_traffic.md).  Keyed by the kernel variant that was profiled: a run whose launcher picked another
+# (the tables of profiles/conv_imtrans_*.md; tests/test_bench_contract.py checks these literals against them).  Keyed
+# by the kernel variant that was profiled: a run whose launcher picked another
 # one, or a configuration that was not profiled, reports null.
 MEASURED_TRAFFIC = {
     # (workload, precision, op): (kernel variant, bytes)
-    ("cfg3", "fp32", "conv"): ("tall16", (56346.0 * 2 + 25088.0) * 1024),        # algorithmic 129.5 MB
-    ("cfg3", "fp32", "imtrans"): (None, (12582.0 * 2 + 100455.8) * 1024),         # algorithmic 128.45 MB
+    ("cfg3", "fp32", "conv"): ("wide48", (56441.5 * 2 + 25088.0) * 1024),        # algorithmic 129.5 MB
+    ("cfg3", "fp32", "imtrans"): (None, (12575.0 * 2 + 100422.5) * 1024),         # algorithmic 128.45 MB
     ("cfg2", "fp32", "conv"): ("tall16", (108090.0 * 2 + 50176.0) * 1024),       # algorithmic 257.2 MB
     ("cfg2", "fp32", "imtrans"): (None, (25126.2 * 2 + 200811.9) * 1024),
     ("cfg4a", "fp32", "conv"): ("short16", (48243.9 * 2 + 12544.0) * 1024),      # algorithmic 68.4 MB
     ("cfg4a", "fp32", "imtrans"): (None, (6432.0 * 2 + 50176.0) * 1024),
     ("cfg4b", "fp32", "conv"): ("short16", (83452.0 * 2 + 8192.0) * 1024),       # algorithmic 58.7 MB
     ("cfg4b", "fp32", "imtrans"): (None, (3175.0 * 2 + 32768.0) * 1024),
-    ("cfg3", "bf16_stored", "conv"): ("stored-ring3", (29943.0 * 2 + 25088.0) * 1024),   # algorithmic 77.6 MB
+    ("cfg3", "bf16_stored", "conv"): ("stored-tall", (30373.5 * 2 + 25088.0) * 1024),    # algorithmic 77.6 MB
     ("cfg3", "bf16_stored", "imtrans"): (None, (12584.0 * 2 + 50176.0) * 1024),
     ("cfg2", "bf16_stored", "conv"): ("stored-ring3", (58798.7 * 2 + 50176.0) * 1024),
     ("cfg2", "bf16_stored", "imtrans"): (None, (25128.0 * 2 + 100352.0) * 1024),
@@ -286,9 +287,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg5", "sweep"],
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg5", "sweep", "layer"],
                     help="cfg1-cfg4b: one layer; cfg5: the whole ResNet-18-var forward (16 Winograd layers), N=128; "
-                         "sweep: the fp32 conv kernel under every tiling over the model's layer shapes and a few others")
+                         "sweep: the fp32 conv kernel under every tiling over the model's layer shapes and a few others; "
+                         "layer: one layer of the shape given with --layer")
+    ap.add_argument("--layer", default="128,14,512,512,0.1", metavar="N,HW,C,K[,density]",
+                    help="shape of --workload layer (input N x HW x HW x C, K filters, N(0,1) input, weights pruned to "
+                         "`density`): e.g. the ResNet-18-var layers at the model's batch, for profiles of one kernel")
     ap.add_argument("--batch", type=int, default=128, help="batch size of the cfg5 forward")
     ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16", "bf16_stored"],
                     help="fp32 (the reference's arithmetic); bf16: GEMM operands rounded to bf16 inside the conv "
@@ -341,6 +346,11 @@ def main():
           getattr(prop, "clock_rate", 0) / 1e3, prop.total_memory / 2 ** 30), file=sys.stderr)
 
     name = args.workload
+    if name == "layer":
+        f = args.layer.split(",")
+        n_, hw_, c_, k_ = (int(v) for v in f[:4])
+        WORKLOADS["layer"] = (n_, hw_, hw_, c_, k_, float(f[4]) if len(f) > 4 else 1.0, "normal")
+        SEEDS["layer"] = 500
     if name == "cfg5":
         return bench_resnet(args, torch, dev)
     if name == "sweep":

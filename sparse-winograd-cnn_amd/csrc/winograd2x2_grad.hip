@@ -22,6 +22,7 @@
 
 #include "swc_common.h"
 #include "winograd2x2_conv_launch.h"
+#include "winograd2x2_dgrad_wide_kernel.h"
 #include "winograd2x2_wgrad_kernel.h"
 
 namespace swc {
@@ -378,8 +379,61 @@ int gemm16_plain(const float *A, const float *Bm, float *Out, size_t P, int Q, s
 using DgradTile = ConvCfg<64, 64, 32, 2, 2, 4>;
 constexpr int kDgradPositions = 2;
 
+// dTI on 48-row x 128-column workgroups that walk all 16 positions (winograd2x2_dgrad_wide_kernel.h): 28x28x128 at
+// batch 64 takes 6.125 tile units per SIMD this way where 64x64 tiles need 6.5 and leave a ragged last round.
+// SWC_ERR_UNSUPPORTED when the shapes do not fit or too few workgroups would run.
+int dgrad_wide(const float *dP, const float *W, float *dTI, size_t M, int C, int K, bool forced, hipStream_t s)
+{
+    if (K % 64 != 0 || C % 128 != 0 || !aligned16(dP) || !aligned16(W) || !aligned16(dTI) || M < 48 || M >= (1ull << 31) ||
+        M * static_cast<size_t>(K > C ? K : C) * 4 >= (1ull << 31) || static_cast<size_t>(C) * K * 4 >= (1ull << 31))
+        return SWC_ERR_UNSUPPORTED;
+    const size_t cus = device_cus(), tiles_n = static_cast<size_t>(C) / 128;
+    auto passes_of = [&](size_t wgs) { return static_cast<double>((wgs + cus - 1) / cus); };
+    // levelled row groups in whole rounds of the chip
+    const size_t gmin = (M + 47) / 48;
+    size_t groups = (gmin * tiles_n + cus - 1) / cus * cus / tiles_n;
+    if (groups < gmin) groups = gmin;
+    size_t rows = (M + groups - 1) / groups;
+    groups = (M + rows - 1) / rows;
+    size_t main_rows = M, extra_wgs = 0;
+    double units = passes_of(groups * tiles_n) * 6.0;
+    // or full 48-row groups in whole rounds, the rest by position: workgroups of 6/16 of a unit each, resident beside
+    // the others
+    size_t g2 = (M / 48) * tiles_n / cus * cus / tiles_n;
+    if (g2 == 0) g2 = M / 48;
+    const size_t left_groups = (M - g2 * 48 + 47) / 48;
+    const double units2 = passes_of(g2 * tiles_n) * 6.0 + passes_of(left_groups * tiles_n * 16) * 6.0 / 16.0;
+    if (left_groups > 0 && units2 < units) {
+        groups = g2;
+        rows = 48;
+        main_rows = g2 * 48;
+        extra_wgs = left_groups * tiles_n * 16;
+        units = units2;
+    }
+    // Against the 64x64-tile kernel (four of its workgroups to a SIMD, any number of tiles): worth it when the
+    // rounds come out nearly full.
+    const double ideal = static_cast<double>(M) * C / 256.0 / (4.0 * cus);  // tile units per SIMD with no rounding at all
+    if (!forced && (units > 1.08 * ideal || groups * tiles_n < cus)) return SWC_ERR_UNSUPPORTED;
+    using Wd = WideDgradCfg;
+    static_assert(2 * Wd::LDS_BYTES <= 160 * 1024, "two workgroups per CU");
+    const size_t n_main = groups * tiles_n;
+    if (n_main + extra_wgs >= (1ull << 29)) return SWC_ERR_BAD_DIMS;
+    conv_dgrad_wide_kernel<<<dim3(static_cast<unsigned>(n_main + extra_wgs)), dim3(Wd::NT), Wd::LDS_BYTES, s>>>(
+        dP, W, dTI, static_cast<unsigned>(M), C, K, static_cast<unsigned>(tiles_n), static_cast<unsigned>(rows),
+        static_cast<unsigned>(main_rows), static_cast<unsigned>(n_main));
+    return check_launch();
+}
+
 int dgrad_own(const float *dP, const float *W, float *dTI, size_t M, int C, int K, hipStream_t s)
 {
+    // swc_winograd2x2_conv_force_tiling applies to the data gradient as well: "wide48" forces the wide kernel where
+    // the shapes allow it, any other name the 64x64-tile kernel.
+    const char *forced = forced_conv_tiling();
+    const bool force_wide = forced != nullptr && std::string_view(forced) == "wide48";
+    if (forced == nullptr || force_wide) {
+        const int st = dgrad_wide(dP, W, dTI, M, C, K, force_wide, s);
+        if (st != SWC_ERR_UNSUPPORTED) return st;
+    }
     // 32-bit offsets: elements within a workgroup's rows of a plane, bytes within a position's weights
     if (static_cast<size_t>(DgradTile::BM) * C >= (1ull << 30) || static_cast<size_t>(C) * K >= (1ull << 30))
         return SWC_ERR_UNSUPPORTED;

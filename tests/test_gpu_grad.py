@@ -102,6 +102,47 @@ def test_conv_grad(oracle, dev, shape):
         assert np.array_equal(a.cpu().numpy(), aw) and np.array_equal(b.cpu().numpy(), bw)
 
 
+@pytest.mark.parametrize("shape", [
+    (8, 14, 14, 128, 128),   # levelled row groups
+    (2, 20, 20, 128, 64),    # 16 full 48-row groups + 2 left-over row tiles: 256 (tile, position) products
+    (2, 2, 197, 128, 64),    # the second left-over tile holds 4 rows
+    (3, 5, 7, 256, 128),     # two column groups, one valid row per workgroup
+    (32, 1, 193, 256, 64),   # two column groups, left-over rows
+])
+def test_conv_grad_data_gradient_on_wide_tiles(oracle, dev, shape):
+    """dTI on the 48-row x 128-column kernel, forced on shapes below the size at which the launcher takes it by
+    itself (swc_winograd2x2_conv_force_tiling("wide48") covers the data gradient as well)."""
+    import swc_hip
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv_grad
+    L = swc_hip.lib()
+    B, nH, nW, C, K = shape
+    rng = np.random.default_rng(34)
+    ti = np.maximum(rng.standard_normal((16, B, nH, nW, C)), 0).astype(np.float32)
+    w = (rng.standard_normal((16, C, K)) * 0.05).astype(np.float32)
+    dy = rng.standard_normal((B, 2 * nH, 2 * nW, K)).astype(np.float32)
+    tii = rng.integers(-3, 4, size=ti.shape).astype(np.float32)
+    wi = rng.integers(-3, 4, size=w.shape).astype(np.float32)
+    dyi = rng.integers(-3, 4, size=dy.shape).astype(np.float32)
+    assert L.swc_winograd2x2_conv_force_tiling(b"wide48") == 0
+    try:
+        dti, dw = winograd2x2_conv_grad(gpu(ti, dev), gpu(w, dev), gpu(dy, dev))
+        a, b = winograd2x2_conv_grad(gpu(tii, dev), gpu(wi, dev), gpu(dyi, dev))
+    finally:
+        assert L.swc_winograd2x2_conv_force_tiling(None) == 0
+    dti_want, dw_want = oracle.conv_grad(ti, w, dy)
+    assert rel_max(dti.cpu().numpy(), dti_want) <= TOL
+    assert rel_max(dw.cpu().numpy(), dw_want) <= TOL
+    aw, bw = oracle.conv_grad(tii, wi, dyi)
+    assert np.array_equal(a.cpu().numpy(), aw) and np.array_equal(b.cpu().numpy(), bw)
+    # the same call with the 64x64-tile kernel forced gives the same values to rounding
+    assert L.swc_winograd2x2_conv_force_tiling(b"ring32") == 0
+    try:
+        dti2, _ = winograd2x2_conv_grad(gpu(ti, dev), gpu(w, dev), gpu(dy, dev))
+    finally:
+        assert L.swc_winograd2x2_conv_force_tiling(None) == 0
+    assert rel_max(dti2.cpu().numpy(), dti_want) <= TOL
+
+
 def test_autograd_through_the_layer(oracle, dev):
     # d/dx and d/dW of sum(g * WinogradConv(WinogradImTrans(x, relu))) against the oracle chain.
     from winograd_conv import WinogradConv
