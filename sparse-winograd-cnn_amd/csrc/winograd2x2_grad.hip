@@ -24,6 +24,7 @@
 #include "winograd2x2_conv_launch.h"
 #include "winograd2x2_dgrad_wide_kernel.h"
 #include "winograd2x2_wgrad_kernel.h"
+#include "winograd2x2_wgrad_wide_kernel.h"
 
 namespace swc {
 namespace {
@@ -456,11 +457,46 @@ int dgrad_own(const float *dP, const float *W, float *dTI, size_t M, int C, int 
 // dTI buffer, which the caller owns, which is at least S*16*C*K floats when S*K <= M, and which is
 // only written (in full) by the dTI GEMM that runs afterwards.  Returns SWC_ERR_UNSUPPORTED when the
 // shapes do not fit the kernel.
+// dW on 128x128 tiles (wgrad_wide_kernel): one workgroup per CU in total, the rows split S ways.
+using WgradWide = WgradWideCfg<16, 3, 2>;
+int wgrad_wide(const float *TI, const float *dP, float *dW, float *scratch, size_t M, int C, int K, hipStream_t s)
+{
+    if (M % WgradWide::BKM != 0 || C % 128 != 0 || K % 128 != 0) return SWC_ERR_UNSUPPORTED;
+    if (static_cast<size_t>(WgradWide::BKM) * C >= (1ull << 29) || static_cast<size_t>(WgradWide::BKM) * K >= (1ull << 29))
+        return SWC_ERR_UNSUPPORTED;  // 32-bit byte offsets within a tile
+    const size_t tiles_c = static_cast<size_t>(C) / 128, tiles_k = static_cast<size_t>(K) / 128;
+    const size_t base = 16 * tiles_c * tiles_k;
+    const size_t steps_total = M / WgradWide::BKM;
+    const size_t cus = device_cus();
+    size_t S = base >= cus ? 1 : (cus + base / 2) / base;
+    if (S > M / K) S = M / K;   // the partial tiles are parked in the dTI buffer: S*16*C*K <= 16*M*C floats
+    if (S > steps_total) S = steps_total;
+    if (S < 1) S = 1;
+    const size_t per = (steps_total + S - 1) / S;
+    S = (steps_total + per - 1) / per;  // no empty split
+    if (S * base >= (1ull << 31)) return SWC_ERR_UNSUPPORTED;
+    const size_t nw = static_cast<size_t>(16) * C * K;
+    wgrad_wide_kernel<WgradWide><<<dim3(static_cast<unsigned>(S * base)), dim3(WgradWide::NT), WgradWide::LDS_BYTES, s>>>(
+        TI, dP, S == 1 ? dW : scratch, M, C, K, static_cast<unsigned>(tiles_c), static_cast<unsigned>(tiles_k),
+        static_cast<unsigned>(per), static_cast<unsigned>(steps_total), nw);
+    int st = check_launch();
+    if (st != SWC_OK || S == 1) return st;
+    const unsigned n4 = static_cast<unsigned>(nw / 4);
+    wgrad_reduce_kernel<<<dim3((n4 + 255) / 256), dim3(256), 0, s>>>(scratch, dW, n4, static_cast<unsigned>(S), nw);
+    return check_launch();
+}
+
 int wgrad_own(const float *TI, const float *dP, float *dW, float *scratch, size_t M, int C, int K, hipStream_t s)
 {
-    if (M % WG_BK != 0 || C % 4 != 0 || K % 4 != 0 || !aligned16(TI) || !aligned16(dP) || !aligned16(dW) ||
-        !aligned16(scratch))
+    if (C % 4 != 0 || K % 4 != 0 || !aligned16(TI) || !aligned16(dP) || !aligned16(dW) || !aligned16(scratch))
         return SWC_ERR_UNSUPPORTED;
+    // "wide48" forces the 128x128 tiles where the shapes allow them, any other forced tiling the 64x64 kernel
+    const char *forced = forced_conv_tiling();
+    if (forced == nullptr || std::string_view(forced) == "wide48") {
+        const int st = wgrad_wide(TI, dP, dW, scratch, M, C, K, s);
+        if (st != SWC_ERR_UNSUPPORTED) return st;
+    }
+    if (M % WG_BK != 0) return SWC_ERR_UNSUPPORTED;
     if (static_cast<size_t>(WG_BK) * C >= (1ull << 29) || static_cast<size_t>(WG_BK) * K >= (1ull << 29))
         return SWC_ERR_UNSUPPORTED;  // 32-bit byte offsets within a tile
     const size_t tiles_c = (static_cast<size_t>(C) + WG_BM - 1) / WG_BM, tiles_k = (static_cast<size_t>(K) + WG_BN - 1) / WG_BN;

@@ -124,15 +124,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
-// dW = sum over splits, ascending, of the partial tiles.  One lane per 4 floats.
+// dW = sum over splits, ascending, of the partial tiles.  One lane per 4 floats; the loads of eight splits are
+// requested before the first of them is added.
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float *__restrict__ part, float *__restrict__ dW,
                                                            unsigned n4, unsigned splits, size_t split_stride)
 {
     const unsigned idx = blockIdx.x * 256 + threadIdx.x;
     if (idx >= n4) return;
-    float4 s = reinterpret_cast<const float4 *>(part)[idx];
-    for (unsigned q = 1; q < splits; ++q) {
-        const float4 v = reinterpret_cast<const float4 *>(part + q * split_stride)[idx];
+    const float4 *p = reinterpret_cast<const float4 *>(part) + idx;
+    const size_t stride4 = split_stride / 4;
+    float4 s = *p;
+    unsigned q = 1;
+    for (; q + 8 <= splits; q += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = p[(q + j) * stride4];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            s.x += v[j].x;
+            s.y += v[j].y;
+            s.z += v[j].z;
+            s.w += v[j].w;
+        }
+    }
+    for (; q < splits; ++q) {
+        const float4 v = p[q * stride4];
         s.x += v.x;
         s.y += v.y;
         s.z += v.z;

@@ -143,6 +143,41 @@ def test_conv_grad_data_gradient_on_wide_tiles(oracle, dev, shape):
     assert rel_max(dti2.cpu().numpy(), dti_want) <= TOL
 
 
+@pytest.mark.parametrize("shape", [
+    (1, 4, 4, 128, 128),     # M = 16: a single step, no split
+    (2, 4, 6, 128, 128),     # M = 48: three steps, no split
+    (4, 8, 9, 128, 128),     # M = 288: two splits of nine steps
+    (2, 8, 17, 128, 256),    # M = 272 = 17 x 16: not a multiple of 32, two filter tiles
+    (8, 8, 13, 256, 128),    # M = 832: six splits, the last one shorter, two channel tiles
+])
+def test_conv_grad_weight_gradient_on_wide_tiles(oracle, dev, shape):
+    """dW on the 128x128-tile kernel (C and K multiples of 128, M a multiple of 16), taken by default and under
+    "wide48"; any other forced tiling runs the 64x64-tile kernel or the plain GEMM on the same shapes."""
+    import swc_hip
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv_grad
+    L = swc_hip.lib()
+    B, nH, nW, C, K = shape
+    rng = np.random.default_rng(35)
+    ti = np.maximum(rng.standard_normal((16, B, nH, nW, C)), 0).astype(np.float32)
+    w = (rng.standard_normal((16, C, K)) * 0.05).astype(np.float32)
+    dy = rng.standard_normal((B, 2 * nH, 2 * nW, K)).astype(np.float32)
+    tii = rng.integers(-3, 4, size=ti.shape).astype(np.float32)
+    wi = rng.integers(-3, 4, size=w.shape).astype(np.float32)
+    dyi = rng.integers(-3, 4, size=dy.shape).astype(np.float32)
+    dti_want, dw_want = oracle.conv_grad(ti, w, dy)
+    aw, bw = oracle.conv_grad(tii, wi, dyi)
+    for forced in (None, b"wide48", b"ring32"):
+        assert L.swc_winograd2x2_conv_force_tiling(forced) == 0
+        try:
+            dti, dw = winograd2x2_conv_grad(gpu(ti, dev), gpu(w, dev), gpu(dy, dev))
+            a, b = winograd2x2_conv_grad(gpu(tii, dev), gpu(wi, dev), gpu(dyi, dev))
+        finally:
+            assert L.swc_winograd2x2_conv_force_tiling(None) == 0
+        assert rel_max(dw.cpu().numpy(), dw_want) <= TOL, forced
+        assert rel_max(dti.cpu().numpy(), dti_want) <= TOL, forced
+        assert np.array_equal(b.cpu().numpy(), bw) and np.array_equal(a.cpu().numpy(), aw), forced
+
+
 def test_autograd_through_the_layer(oracle, dev):
     # d/dx and d/dW of sum(g * WinogradConv(WinogradImTrans(x, relu))) against the oracle chain.
     from winograd_conv import WinogradConv
