@@ -148,7 +148,7 @@ int launch_bf16_stored(const unsigned short *Input16, const unsigned short *Weig
     struct Tag {};
     const int st = raise_lds_limit<Tag>(reinterpret_cast<const void *>(conv_bf16_stored_kernel<Hb, GROUPS>), lds_bytes);
     if (st != SWC_OK) return st;
-    conv_bf16_stored_kernel<Hb, GROUPS><<<dim3(static_cast<unsigned>(tiles_m * tiles_n)), dim3(256 * GROUPS), lds_bytes, s>>>(
+    conv_bf16_stored_kernel<Hb, GROUPS><<<dim3(static_cast<unsigned>(tiles_m * tiles_n)), dim3(64 * Hb::GW * GROUPS), lds_bytes, s>>>(
         Input16, Weight16t, Output, M, C, K, nH, nW, static_cast<unsigned>(tiles_n), static_cast<unsigned>(rows_per_wg), ep);
     return check_launch();
 }
@@ -170,6 +170,7 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
     using Deep = HbCfg<64, 4, 2>;   // 4-deep ring, up to two workgroups per CU
     using Wide = HbCfg<64, 3, 3>;   // 3-deep ring, up to three workgroups per CU
     using Split = HbCfg<64, 3, 2>;  // two groups of waves per workgroup, a 3-deep ring each
+    using Quad = HbCfg<64, 3, 2, 32>;  // 32-row tiles, four groups of two waves per workgroup, a 3-deep ring each
     if (C % Deep::BK != 0 || !aligned16(Input16) || !aligned16(Weight16t) || static_cast<size_t>(HB_BM) * C >= (1ull << 30))
         return SWC_ERR_UNSUPPORTED;
     const size_t tiles_n = (static_cast<size_t>(K) + HB_BN - 1) / HB_BN;
@@ -211,6 +212,14 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
     // A grid of full tiles that leaves every CU with one workgroup at most: the launch then lasts as long as one
     // workgroup's chain of steps, and splitting the 16 positions over two groups of waves halves the chain
     // (7x7x512 at batch 64: 30.7 us against 37.1; 14x14x256: 19.9 against 22.9).
+    // Fewer tiles still, so that 32-row tiles also leave every CU with one workgroup at most, and long positions
+    // (four steps or more): four groups of two waves, four positions each.  Such a launch is bound by what one CU
+    // can copy into its LDS (about 40 bytes a clock), and twice the workgroups on twice the CUs move 1.5 times the
+    // bytes in all: 7x7x512 at batch 64 23.8 us against 27.1.
+    if ((M + 31) / 32 * tiles_n <= cus && C >= 4 * Quad::BK) {
+        note_conv_kernel("stored-split4");
+        return launch_bf16_stored<Quad, 4>(Input16, Weight16t, Output, M, C, K, nH, nW, 32, tiles_n, ep, s);
+    }
     if ((M + HB_BM - 1) / HB_BM * tiles_n <= cus) {
         note_conv_kernel("stored-split");
         return launch_bf16_stored<Split, 2>(Input16, Weight16t, Output, M, C, K, nH, nW, HB_BM, tiles_n, ep, s);

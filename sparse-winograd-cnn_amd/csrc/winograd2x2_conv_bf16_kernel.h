@@ -21,54 +21,60 @@ namespace {
 constexpr int HB_BM = 64, HB_BN = 64;  // tile of the [M,K] plane; 4 waves, 2x2, 32x32 each
 using HbStoreCfg = ConvCfg<HB_BM, HB_BN, 32, 2, 2>;
 
-// BK channels per step (a tile row is BK*2 bytes = CH chunks of 16), NSTAGE ring slots, OCC waves per SIMD.
-template <int BK_, int NSTAGE_, int OCC_>
+// BK channels per step (a tile row is BK*2 bytes = CH chunks of 16), NSTAGE ring slots, OCC waves per SIMD, BM
+// rows per tile: 64 (four waves, 2x2) or 32 (two waves side by side).
+template <int BK_, int NSTAGE_, int OCC_, int BM_ = HB_BM>
 struct HbCfg {
-    static constexpr int BK = BK_, NSTAGE = NSTAGE_, OCC = OCC_;
+    static constexpr int BK = BK_, NSTAGE = NSTAGE_, OCC = OCC_, BM = BM_;
+    static constexpr int GW = BM / 16;                   // waves of a group: one per 32x32 part of the BM x 64 tile
     static constexpr int CH = BK / 8;                    // 16-byte chunks per tile row
     static constexpr int ROWS_PER_COPY = 64 / CH;        // rows one wave-wide copy (1 KiB) covers
-    static constexpr int TILE_BYTES = 64 * BK * 2;       // per operand
-    static constexpr int TILE_COPIES = TILE_BYTES / 1024;
-    static constexpr int PER_WAVE = TILE_COPIES / 4;     // copies of each tile per wave and step
-    static constexpr int COPIES = 2 * PER_WAVE;          // per thread and step
-    static constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+    static constexpr int A_BYTES = BM * BK * 2;          // activation tile
+    static constexpr int TILE_BYTES = 64 * BK * 2;       // weight tile
+    static constexpr int PER_WAVE_A = A_BYTES / 1024 / GW, PER_WAVE = TILE_BYTES / 1024 / GW;  // copies per wave and step
+    static constexpr int COPIES = PER_WAVE_A + PER_WAVE; // per thread and step
+    static constexpr int STAGE_BYTES = A_BYTES + TILE_BYTES;
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
     static constexpr int NMFMA = BK / 16;                // MFMAs per step and wave
+    using Store = ConvCfg<BM, HB_BN, 32, BM / 32, 2>;
     static_assert(BK == 32 || BK == 64 || BK == 128, "a tile row is 4, 8 or 16 chunks");
-    static_assert(TILE_COPIES % 4 == 0, "every wave issues the same number of copies");
+    static_assert(BM == 64 || BM == 32, "four or two waves per group");
+    static_assert(A_BYTES / 1024 % GW == 0 && TILE_BYTES / 1024 % GW == 0, "every wave issues the same number of copies");
     static_assert((NSTAGE - 2) * COPIES < 64, "vmcnt range");
 };
 
 // Requires C % BK == 0 and 16-byte aligned TI16 / Wt16.  M < 2^31.  grid.x = ceil(M / rows_per_wg) * tiles_n.
 //
-// GROUPS = 2: a workgroup is two groups of four waves that share the tile and split its 16 positions, 0-7 and
-// 8-15, each group with its own ring; at the end the second group hands its four partial output tiles to the first
-// through LDS, which adds them to its own and stores.  For grids that leave a CU with one workgroup: the time
-// of such a launch is one workgroup's chain of dependent steps (wait, barrier, copies, LDS reads, four MFMAs), and
-// two chains of half the length run side by side on the same SIMDs.  The sum of the transform is then taken as
-// (positions 0-7) + (positions 8-15) instead of in one ascending chain.  Needs 2*LDS_BYTES of LDS.
+// GROUPS = 2 or 4: a workgroup is that many groups of waves that share the tile and split its 16 positions (0-7
+// and 8-15, or four each), each group with its own ring; at the end the other groups hand their four partial
+// output tiles to the first through LDS, which adds them to its own in ascending group order and stores.  For
+// grids that leave a CU with one workgroup: the time of such a launch is one workgroup's chain of dependent
+// steps (wait, barrier, copies, LDS reads, four MFMAs), and chains of a half or a quarter of the length run side by
+// side on the same SIMDs.  The sum of the transform is then taken group by group instead of in one ascending
+// chain.  Needs GROUPS*LDS_BYTES of LDS.
 template <typename Cfg, int GROUPS = 1>
-__global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_bf16_stored_kernel(
+__global__ __launch_bounds__(64 * Cfg::GW * GROUPS) __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void conv_bf16_stored_kernel(
     const unsigned short *__restrict__ TI16, const unsigned short *__restrict__ Wt16, float *__restrict__ Out, size_t M,
     int C, int K, int nH, int nW, unsigned tiles_n, unsigned rows_per_wg, ConvEpilogue ep)
 {
     constexpr int BK = Cfg::BK, NSTAGE = Cfg::NSTAGE, CH = Cfg::CH, RPC = Cfg::ROWS_PER_COPY, PW = Cfg::PER_WAVE;
+    constexpr int PWA = Cfg::PER_WAVE_A, GW = Cfg::GW;
     constexpr int ROW_BYTES = BK * 2;
     constexpr int RPL = ROW_BYTES >= 256 ? 1 : 256 / ROW_BYTES;  // tile rows per 256 bytes of LDS (one pass over its banks)
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem_b[];
 
     const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
-    // A workgroup takes rows_per_wg <= HB_BM rows (the launcher levels the load over the CUs with it).
+    // A workgroup takes rows_per_wg <= BM rows (the launcher levels the load over the CUs with it).
     const size_t m0 = static_cast<size_t>(lid / tiles_n) * rows_per_wg;
     const int n0 = static_cast<int>(lid % tiles_n) * HB_BN;
     const unsigned rows_valid = static_cast<unsigned>(M - m0 < rows_per_wg ? M - m0 : rows_per_wg);
     const unsigned cols_valid = static_cast<unsigned>(K - n0 < HB_BN ? K - n0 : HB_BN);
 
-    static_assert(GROUPS == 1 || GROUPS == 2, "one or two groups of four waves");
+    static_assert(GROUPS == 1 || GROUPS == 2 || GROUPS == 4, "one, two or four groups of waves");
     constexpr int NPOS = 16 / GROUPS;  // positions per group
     const int tid = threadIdx.x, lane = tid & 63;
     const unsigned wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const unsigned group = wave_wg >> 2, wave = wave_wg & 3;  // wave: index within the group
+    const unsigned group = wave_wg / GW, wave = wave_wg % GW;  // wave: index within the group
     const int li = lane & 31, lg = lane >> 5;
     const int wm0 = static_cast<int>(wave >> 1) * 32, wn0 = static_cast<int>(wave & 1) * 32;
     const int nkc = C / BK;
@@ -76,15 +82,22 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(Cf
 
     // ---- copies: wave-copy wl of a tile covers its rows RPC*wl .. RPC*wl+RPC-1 (1 KiB) ------------------
     // Rows beyond the valid ones re-read the last valid row; they only reach outputs that are never stored.
-    unsigned a_voff[PW], b_voff[PW], t_lds[PW];
+    unsigned a_voff[PWA], b_voff[PW], ta_lds[PWA], tb_lds[PW];
+#pragma unroll
+    for (int q = 0; q < PWA; ++q) {
+        const unsigned wl = wave * PWA + q;
+        const unsigned row = RPC * wl + lane / CH, slot = lane % CH, chunk = slot ^ ((row / RPL) % CH);
+        const unsigned ra = row < rows_valid ? row : rows_valid - 1;
+        a_voff[q] = (ra * static_cast<unsigned>(C) + chunk * 8) * 2u;
+        ta_lds[q] = wl * 1024u;
+    }
 #pragma unroll
     for (int q = 0; q < PW; ++q) {
         const unsigned wl = wave * PW + q;
         const unsigned row = RPC * wl + lane / CH, slot = lane % CH, chunk = slot ^ ((row / RPL) % CH);
-        const unsigned ra = row < rows_valid ? row : rows_valid - 1, rb = row < cols_valid ? row : cols_valid - 1;
-        a_voff[q] = (ra * static_cast<unsigned>(C) + chunk * 8) * 2u;
+        const unsigned rb = row < cols_valid ? row : cols_valid - 1;
         b_voff[q] = (rb * static_cast<unsigned>(C) + chunk * 8) * 2u;
-        t_lds[q] = wl * 1024u;
+        tb_lds[q] = Cfg::A_BYTES + wl * 1024u;
     }
     const unsigned smem_base = lds_address(smem_g);
     const size_t a_pos_stride = M * static_cast<size_t>(C), b_pos_stride = static_cast<size_t>(K) * C;
@@ -101,10 +114,9 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(Cf
     // Every thread issues exactly Cfg::COPIES copies per call.
     auto issue = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int q = 0; q < PW; ++q) async_copy16(reinterpret_cast<const float *>(a_next), a_voff[q], dst_next + t_lds[q]);
+        for (int q = 0; q < PWA; ++q) async_copy16(reinterpret_cast<const float *>(a_next), a_voff[q], dst_next + ta_lds[q]);
 #pragma unroll
-        for (int q = 0; q < PW; ++q)
-            async_copy16(reinterpret_cast<const float *>(b_next), b_voff[q], dst_next + Cfg::TILE_BYTES + t_lds[q]);
+        for (int q = 0; q < PW; ++q) async_copy16(reinterpret_cast<const float *>(b_next), b_voff[q], dst_next + tb_lds[q]);
         const bool last_chunk = --kc_left == 0;
         kc_left = last_chunk ? nkc : kc_left;
         a_next += last_chunk ? a_jump : static_cast<size_t>(BK);
@@ -131,7 +143,7 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(Cf
     for (int h = 0; h < Cfg::NMFMA; ++h) {
         const unsigned ra = wm0 + li, rb = wn0 + li;
         a_off[h] = ra * ROW_BYTES + (((2 * h + lg) ^ ((ra / RPL) % CH)) * 16u);
-        b_off[h] = Cfg::TILE_BYTES + rb * ROW_BYTES + (((2 * h + lg) ^ ((rb / RPL) % CH)) * 16u);
+        b_off[h] = Cfg::A_BYTES + rb * ROW_BYTES + (((2 * h + lg) ^ ((rb / RPL) % CH)) * 16u);
     }
     unsigned st_next = 0;  // byte offset of the ring slot whose operands are fetched next
 
@@ -200,34 +212,50 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(Cf
             }
         });
     };
-    if (GROUPS == 1 || group == 0)
+    if constexpr (GROUPS == 1) {
         positions(std::integral_constant<int, 0>{});
-    else
-        positions(std::integral_constant<int, 16 - NPOS>{});
+    } else if constexpr (GROUPS == 2) {
+        if (group == 0)
+            positions(std::integral_constant<int, 0>{});
+        else
+            positions(std::integral_constant<int, 8>{});
+    } else {
+        if (group == 0)
+            positions(std::integral_constant<int, 0>{});
+        else if (group == 1)
+            positions(std::integral_constant<int, 4>{});
+        else if (group == 2)
+            positions(std::integral_constant<int, 8>{});
+        else
+            positions(std::integral_constant<int, 12>{});
+    }
     wait_vmcnt<0>();  // the surplus copies must land before the workgroup's LDS is handed on
 
-    if constexpr (GROUPS == 2) {
-        // The second group's partial sums go through LDS, [j][register][thread of the group] (64 KiB: the rings are
-        // idle by now), and are added to the first group's, which then stores alone.
-        static_assert(2 * Cfg::LDS_BYTES >= 4 * 16 * 256 * 4, "the rings hold the four partial tiles");
+    if constexpr (GROUPS > 1) {
+        // The other groups' partial sums go through LDS, [group][j][register][thread of the group] (the rings are idle
+        // by now), and are added to the first group's in ascending group order; the first group then stores alone.
+        constexpr int TG = 64 * GW;  // threads of a group
+        static_assert(GROUPS * Cfg::LDS_BYTES >= (GROUPS - 1) * 4 * 16 * TG * 4, "the rings hold the partial tiles");
         float *const xch = reinterpret_cast<float *>(smem_b);
-        const int t = tid & 255;
+        const int t = tid % TG;
         __builtin_amdgcn_s_waitcnt(0xc07f);
         __builtin_amdgcn_s_barrier();  // every wave has finished reading its ring
-        if (group == 1) {
+        if (group != 0) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) xch[(j * 16 + r) * 256 + t] = Y[j][0][0][r];
+                for (int r = 0; r < 16; ++r) xch[(((group - 1) * 4 + j) * 16 + r) * TG + t] = Y[j][0][0][r];
         }
         __syncthreads();
-        if (group == 1) return;
+        if (group != 0) return;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int g = 0; g < GROUPS - 1; ++g)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) Y[j][0][0][r] += xch[(j * 16 + r) * 256 + t];
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) Y[j][0][0][r] += xch[((g * 4 + j) * 16 + r) * TG + t];
     }
-    store_output<HbStoreCfg>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
+    store_output<typename Cfg::Store>(Y, Out, rows_valid, K, nW, m0, n0, wm0, wn0, li, lg, ep);
 }
 
 // W [16,C,K] fp32 -> Wt16 [16,K,C] bf16 (round to nearest even).  One lane per output element.

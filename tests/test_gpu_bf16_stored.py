@@ -87,14 +87,57 @@ def test_conv_over_bf16_operands(oracle, dev, shape):
     same = winograd2x2_conv(gpu(ti, dev), gpu(w, dev), precision="bf16").cpu().numpy()
     assert rel_max(got, same) <= TOL
     # grids that leave every CU with one workgroup at most (all of these on an MI355X): two groups of waves split
-    # the positions
+    # the positions, or four groups on 32-row tiles where those also fit the CUs and a position has four steps or more
     import swc_hip
     winograd2x2_conv(ti_gpu, gpu(w, dev))
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
     tiles = -(-B * nH * nW // 64) * -(-K // 64)
-    if tiles <= torch.cuda.get_device_properties(dev).multi_processor_count:
+    tiles32 = -(-B * nH * nW // 32) * -(-K // 64)
+    if tiles32 <= cus and C >= 256:
+        assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() == b"stored-split4"
+    elif tiles <= cus:
         assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() == b"stored-split"
     else:
         assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() in (b"stored-ring3", b"stored-ring4")
+
+
+@pytest.mark.parametrize("shape", [
+    (64, 4, 4, 512, 512),    # config 4b: 32 x 8 workgroups of 32 rows, eight steps per position
+    (3, 5, 7, 256, 96),      # M = 105: the last row group holds 9 rows; the second column group 32 columns
+    (1, 1, 1, 320, 4),       # one row, four columns, five steps per position
+    (2, 9, 9, 1024, 192),    # sixteen steps per position
+])
+def test_stored_split4_kernel(oracle, dev, shape):
+    """Small grids of long positions run `stored-split4` (32-row tiles, four groups of two waves, four positions
+    each, partial sums added group by group): values against the oracle fed the same bf16 operands, exactly on
+    integers, and the epilogue's arithmetic exactly."""
+    import swc_hip
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv, winograd2x2_weights_bf16
+    B, nH, nW, C, K = shape
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    if -(-B * nH * nW // 32) * -(-K // 64) > cus:
+        pytest.skip("this device has too few CUs for the shape to take one 32-row tile per CU")
+    rng = np.random.default_rng(68)
+    ti = np.maximum(rng.standard_normal((16, B, nH, nW, C)), 0).astype(np.float32)
+    w = (rng.standard_normal((16, C, K)) * 0.05).astype(np.float32)
+    ti16, w16 = oracle.round_bf16(ti), oracle.round_bf16(w)
+    ti_gpu, w_gpu = gpu(ti16, dev).to(torch.bfloat16), winograd2x2_weights_bf16(gpu(w, dev))
+    got = winograd2x2_conv(ti_gpu, w_gpu).cpu().numpy()
+    assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() == b"stored-split4"
+    want = oracle.conv(ti16, w16, acc64=True)
+    assert got.shape == want.shape
+    assert rel_max(got, want) <= TOL
+    ti_i = rng.integers(-3, 4, size=ti.shape).astype(np.float32)
+    w_i = rng.integers(-3, 4, size=w.shape).astype(np.float32)
+    got_i = winograd2x2_conv(gpu(ti_i, dev).to(torch.bfloat16), gpu(w_i, dev)).cpu().numpy()
+    assert np.array_equal(got_i, oracle.conv(ti_i, w_i))
+    scale = (0.5 + rng.random(K)).astype(np.float32) * rng.choice([-1, 1], K).astype(np.float32)
+    shift = rng.standard_normal(K).astype(np.float32)
+    res = rng.standard_normal(want.shape).astype(np.float32)
+    got2 = winograd2x2_conv(ti_gpu, w_gpu, scale=gpu(scale, dev), shift=gpu(shift, dev), residual=gpu(res, dev)).cpu().numpy()
+    assert np.array_equal(got2, oracle.affine(got, scale, shift) + res)
+    got3 = winograd2x2_conv(ti_gpu, w_gpu, residual=gpu(res, dev), residual_relu=True).cpu().numpy()
+    assert np.array_equal(got3, got + np.maximum(res, 0))
 
 
 @pytest.mark.parametrize("shape", [

@@ -187,6 +187,8 @@ def test_layers_at_batch_128(oracle, hw, C, K, precision):
         tiles = -(-M // 64) * -(-K // 64)
         if C in (128, 256, 512) and K % 64 == 0 and -(-M // 128) * (K // 64) * 4 >= 3 * props.multi_processor_count:
             assert kernel == "stored-tall", kernel      # enough 128-row x 64-column tiles to go round
+        elif -(-M // 32) * -(-K // 64) <= props.multi_processor_count and C >= 256:
+            assert kernel == "stored-split4", kernel
         elif tiles <= props.multi_processor_count:
             assert kernel == "stored-split", kernel
         else:
