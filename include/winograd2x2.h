@@ -49,8 +49,9 @@ SWC_API const char *swc_version(void);
  * (small grids: the 16 positions of a tile split over two groups of waves, whose partial sums are added at the
  * end) / "stored-split4" (smaller grids still: 32-row tiles, four groups of waves) / "stored-tall" (128x64
  * tiles for C = 128, 256 or 512 on grids that fill the device).  Which one runs depends only on the shapes,
- * pointer alignment and the device's CU count and L2 size; all give the same results to within the order of the fp32 summations ("wide48" and "stored-tall" also add the nine terms of an output
- * in another order than the rest: 1e-6 relative, exact on integer-valued data). */
+ * pointer alignment and the device's CU count and L2 size; all give the same results to within the order of
+ * the fp32 summations ("wide48" and "stored-tall" also add the nine terms of an output in another order than
+ * the rest: 1e-6 relative, exact on integer-valued data). */
 SWC_API const char *swc_winograd2x2_conv_last_kernel(void);
 /* Diagnostic with no counterpart in the reference, for benchmarks and tests that compare the tilings: makes
  * the calling thread's later swc_winograd2x2_conv calls
