@@ -48,7 +48,7 @@ SWC_API const char *swc_version(void);
  * bf16-stored operands "stored-ring3" / "stored-ring4" (64x64 tiles, 3- / 4-deep copy ring) / "stored-split"
  * (small grids: the 16 positions of a tile split over two groups of waves, whose partial sums are added at the
  * end) / "stored-split4" (smaller grids still: 32-row tiles, four groups of waves) / "stored-tall" (128x64
- * tiles for C = 128, 256 or 512 on grids that fill the device).  Which one runs depends only on the shapes,
+ * tiles for C = 64, 128, 256 or 512 on grids that fill the device).  Which one runs depends only on the shapes,
  * pointer alignment and the device's CU count and L2 size; all give the same results to within the order of
  * the fp32 summations ("wide48" and "stored-tall" also add the nine terms of an output in another order than
  * the rest: 1e-6 relative, exact on integer-valued data). */

@@ -190,7 +190,7 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
     ep.residual = Residual;
     ep.residual_relu = residual_relu != 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // Layers of 128, 256 or 512 channels with enough 128-row x 64-column tiles for three quarters of the CUs: the
+    // Layers of 64, 128, 256 or 512 channels with enough 128-row x 64-column tiles for three quarters of the CUs: the
     // tall tiles (twice the matrix work per byte through LDS, which bounds these layers: 14x14 at batch 128,
     // 512 -> 512 77 us against 100, 28x28, 128 -> 128 27 against 35; with a residual to add 35 against 58).  With more
     // tiles than CUs two workgroups share a CU and the rows are levelled over whole rounds of them.

@@ -1,5 +1,5 @@
 // Launches of the stored-tall kernel (winograd2x2_conv_bf16_tall_kernel.h), the bf16-stored convolution's form for
-// layers of 128, 256 or 512 input channels with enough 128-row x 64-column tiles to go round the CUs.  A translation
+// layers of 64, 128, 256 or 512 input channels with enough 128-row x 64-column tiles to go round the CUs.  A translation
 // unit of its own: its instantiations take minutes to compile.  Part of what stands in for
 // Winograd2x2ConvComputeLauncher (winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_cuda.cu.cc:65-93) when the
 // transformed activations are held as bf16.
@@ -29,7 +29,7 @@ int launch_tall_as(const unsigned short *TI16, const unsigned short *Wt16, float
 
 bool bf16_tall_eligible(const void *TI16, const void *Wt16, size_t M, int C, int K)
 {
-    return (C == 128 || C == 256 || C == 512) && K % 64 == 0 && aligned16(TI16) && aligned16(Wt16) && M < (1ull << 31) &&
+    return (C == 64 || C == 128 || C == 256 || C == 512) && K % 64 == 0 && aligned16(TI16) && aligned16(Wt16) && M < (1ull << 31) &&
            M * 16 * static_cast<size_t>(K) < (1ull << 31);
 }
 
@@ -45,6 +45,9 @@ int launch_bf16_tall(const unsigned short *TI16, const unsigned short *Wt16, flo
     ep.residual_relu = residual_relu;
     const bool epi = scale != nullptr || residual != nullptr;
     switch (C / 64) {
+        case 1:
+            return epi ? launch_tall_as<1, true>(TI16, Wt16, Out, M, K, nW, rows_per_wg, ep, stream)
+                       : launch_tall_as<1, false>(TI16, Wt16, Out, M, K, nW, rows_per_wg, ep, stream);
         case 2:
             return epi ? launch_tall_as<2, true>(TI16, Wt16, Out, M, K, nW, rows_per_wg, ep, stream)
                        : launch_tall_as<2, false>(TI16, Wt16, Out, M, K, nW, rows_per_wg, ep, stream);

@@ -1,4 +1,4 @@
-// "stored-tall": the bf16-stored convolution for layers with many channels (device code).  Same contract as
+// "stored-tall": the bf16-stored convolution for layers of 64, 128, 256 or 512 channels (device code).  Same contract as
 // conv_bf16_stored_kernel (winograd2x2_conv_bf16_kernel.h): TI as bf16 [16,M,C], weights as bf16 [16,K,C], fp32
 // accumulation, fp32 output transform and output.
 //
@@ -65,10 +65,11 @@ struct TallCfg {
     static constexpr int LDS_BYTES = RING_AT + RING_BYTES;
     static constexpr int NA = A_BYTES / 1024 / 4, NB = B_BYTES / 1024 / 4, LPS = NA + NB;  // copies per wave and step
     static constexpr int PLANE_STORES = TM * 16;          // store instructions of one output plane per wave
-    // A position that stores a plane does its vector work in its first steps and the stores in its last ones.
+    // A position that stores a plane does its vector work in its first steps and the stores in its last ones; a
+    // position of a single step in the first half of the step and in the second.
     static constexpr int STORE_STEPS = NKC >= 2 ? NKC / 2 : 1;
     static constexpr int STORES_PER_STEP = PLANE_STORES / STORE_STEPS;
-    static_assert(NKC == 2 || NKC == 4 || NKC == 8, "128, 256 or 512 channels");
+    static_assert(NKC == 1 || NKC == 2 || NKC == 4 || NKC == 8, "64, 128, 256 or 512 channels");
     static_assert(BM * 4 <= RING_AT && (NKC - 1) * 128 <= RING_AT, "the copies' M0 values stay non-negative");
     static_assert((NA - 1) * 1024 + (NKC - 1) * 128 < 4096, "immediate offsets of the copies");
     static_assert(LPS + STORES_PER_STEP < 64, "vmcnt range");
@@ -278,13 +279,21 @@ __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::OCC, T
         constexpr int n_ops = (kWideOps[q][0][0] != 0) + (kWideOps[q][1][0] != 0);
         constexpr int n_units = n_ops * TM * 4;
         // MFMA slots of the position over which the vector work is spread: all of them, or those of the steps
-        // before the ones that store.
-        constexpr int ride_slots = (store_plane >= 0 ? NKC - T::STORE_STEPS : NKC) * 4 * TM;
+        // before the ones that store (of the half step before the half that stores).
+        constexpr bool one_step = NKC == 1;
+        constexpr int ride_slots = store_plane < 0 ? NKC * 4 * TM : one_step ? 2 * TM : (NKC - T::STORE_STEPS) * 4 * TM;
         constexpr bool stores_here = store_plane >= 0 && kc >= NKC - T::STORE_STEPS;
-        // Stores of the previous step and of this one are younger than the copies of the tile waited for.
+        // Operations issued after the copies of the tile waited for (the next step's) and before the wait: the
+        // copies of the step after it, and stores.  With several steps per position: those of the previous step and of
+        // this one.  With one step per position a step stores in its second half: the last quarter of the step two back
+        // (issued behind that step's copies), all of the previous step, half of this one.
+        auto stores_at = [](int qq) constexpr { return T::EARLY && qq >= 0 && kWideStoreAt[qq >= 0 ? qq : 0] >= 0; };
         constexpr int prev_q = kc > 0 ? q : q - 1, prev_kc = kc > 0 ? kc - 1 : NKC - 1;
-        constexpr bool stores_before =
-            T::EARLY && prev_q >= 0 && kWideStoreAt[prev_q >= 0 ? prev_q : 0] >= 0 && prev_kc >= NKC - T::STORE_STEPS;
+        constexpr bool stores_before = stores_at(prev_q) && prev_kc >= NKC - T::STORE_STEPS;
+        constexpr int younger_stores =
+            one_step ? (stores_at(q - 2) ? T::STORES_PER_STEP / 4 : 0) + (stores_at(q - 1) ? T::STORES_PER_STEP : 0) +
+                           (stores_here ? T::STORES_PER_STEP / 2 : 0)
+                     : (stores_before ? T::STORES_PER_STEP : 0) + (stores_here ? T::STORES_PER_STEP : 0);
         // The step's eight MFMAs, group h = i / 2, tile tm = i % 2; what else a wave has to issue goes between them.
         static_for<4 * TM>([&](auto i_tag) __attribute__((always_inline)) {
             constexpr int i = decltype(i_tag)::value, h = i / TM, tm = i % TM;
@@ -294,13 +303,15 @@ __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::OCC, T
 #pragma unroll
             for (int u = 0; u < n_units; ++u)
                 if (ride_slots > 0 && u * ride_slots / (n_units > 0 ? n_units : 1) == slot_in_pos) ride_unit(q_tag, u);
-            if constexpr (stores_here && h < 2) {
-                // this step's share of the plane's 8 quarters (TM tiles x 4), dealt over its first four slots
+            if constexpr (stores_here && (one_step ? h >= 2 : h < 2)) {
+                // this step's share of the plane's 8 quarters (TM tiles x 4), dealt over its first four slots (over
+                // its last four when the position is this one step and the vector work fills the first four)
                 constexpr int quarters_per_step = T::STORES_PER_STEP / 4;
                 constexpr int first_quarter = (kc - (NKC - T::STORE_STEPS)) * quarters_per_step;
+                constexpr int i_store = one_step ? i - 2 * TM : i;
 #pragma unroll
                 for (int w = 0; w < quarters_per_step; ++w)
-                    if (w * 4 / quarters_per_step == i) {
+                    if (w * 4 / quarters_per_step == i_store) {
                         const int qu = first_quarter + w;
                         store_quarter(store_plane, qu / 4, qu % 4, no_residual);
                     }
@@ -309,7 +320,7 @@ __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::OCC, T
                 if constexpr (h == 2) {
                     // The next step's tile has landed once only what was issued after its copies is outstanding:
                     // the copies of the step after it and the stores of the previous step and of this one.
-                    constexpr int n = LPS + (stores_before ? T::STORES_PER_STEP : 0) + (stores_here ? T::STORES_PER_STEP : 0);
+                    constexpr int n = LPS + younger_stores;
                     wait_vmcnt<(n < 63 ? n : 63)>();  // the counter's range; waiting for fewer outstanding operations is always safe
                     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS reads of this step are done
                     __builtin_amdgcn_s_barrier();

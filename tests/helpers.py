@@ -79,3 +79,16 @@ def rel_l1(a, b):
     b = np.asarray(b, dtype=np.float64)
     den = np.sum(np.abs(a)) + np.sum(np.abs(b))
     return float(np.sum(np.abs(a - b)) / (den if den > 0 else 1.0))
+
+
+def expected_stored_launch(M, C, K, cus, l2_bytes):
+    """The launch form swc_winograd2x2_conv_bf16in picks for tile rows M, channels C, filters K on a device with
+    `cus` compute units and L2s of `l2_bytes` (the rules of its launcher, restated), as a one-element tuple."""
+    ceil = lambda a, b: -(-a // b)
+    if C in (64, 128, 256, 512) and K % 64 == 0 and ceil(M, 128) * (K // 64) * 4 >= 3 * cus:
+        return ("stored-tall",)
+    if ceil(M, 32) * ceil(K, 64) <= cus and C >= 256:
+        return ("stored-split4",)
+    if ceil(M, 64) * ceil(K, 64) <= cus:
+        return ("stored-split",)
+    return ("stored-ring4",) if 16 * C * K * 2 >= l2_bytes else ("stored-ring3",)

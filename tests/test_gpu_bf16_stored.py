@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import rel_max
+from helpers import expected_stored_launch, rel_max
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4
@@ -86,19 +86,12 @@ def test_conv_over_bf16_operands(oracle, dev, shape):
     # the same values as the kernel that rounds fp32 operands in its registers
     same = winograd2x2_conv(gpu(ti, dev), gpu(w, dev), precision="bf16").cpu().numpy()
     assert rel_max(got, same) <= TOL
-    # grids that leave every CU with one workgroup at most (all of these on an MI355X): two groups of waves split
-    # the positions, or four groups on 32-row tiles where those also fit the CUs and a position has four steps or more
+    # which launch form ran: small grids split the positions over groups of waves, large ones take the tall tiles
     import swc_hip
     winograd2x2_conv(ti_gpu, gpu(w, dev))
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    tiles = -(-B * nH * nW // 64) * -(-K // 64)
-    tiles32 = -(-B * nH * nW // 32) * -(-K // 64)
-    if tiles32 <= cus and C >= 256:
-        assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() == b"stored-split4"
-    elif tiles <= cus:
-        assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() == b"stored-split"
-    else:
-        assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() in (b"stored-ring3", b"stored-ring4")
+    props = torch.cuda.get_device_properties(dev)
+    want_launch = expected_stored_launch(B * nH * nW, C, K, props.multi_processor_count, props.L2_cache_size)
+    assert swc_hip.lib().swc_winograd2x2_conv_last_kernel().decode() in want_launch
 
 
 @pytest.mark.parametrize("shape", [
@@ -142,12 +135,14 @@ def test_stored_split4_kernel(oracle, dev, shape):
 
 @pytest.mark.parametrize("shape", [
     (6, 16, 16, 128, 1024),   # 12 x 16 tiles of 128 rows x 64 columns
+    (25, 20, 20, 64, 256),    # 64 channels: a position is a single step (vector work and stores share it)
+    (26, 31, 31, 64, 64),     # M = 24 986: levelled rows, one column group
     (3, 20, 25, 256, 1024),   # M = 1500: the last row group holds 92 rows
     (2, 16, 24, 512, 2048),   # 512 channels: eight steps per position
     (4, 25, 25, 128, 1024),   # more tiles than CUs: rows levelled over whole rounds (79 per workgroup on an MI355X)
 ])
 def test_stored_tall_kernel(oracle, dev, shape):
-    """Layers of 128, 256 or 512 channels with enough tiles for the chip run `stored-tall` (128-row x 64-column
+    """Layers of 64, 128, 256 or 512 channels with enough tiles for the chip run `stored-tall` (128-row x 64-column
     workgroups, the output transform in the sum/difference association): values against the oracle fed the same
     bf16 operands, exactly on integers (every sign and the scatter), and the epilogue's arithmetic exactly."""
     import swc_hip

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import rel_l1, rel_max
+from helpers import expected_stored_launch, rel_l1, rel_max
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4
@@ -56,10 +56,7 @@ def test_config4_full_size(oracle, layer):
     assert np.array_equal(ti16.view(torch.int16).cpu().numpy().view(np.uint16), oracle.bf16_bits(ti_want))
     got = winograd2x2_conv(ti16, gpu(w, dev)).cpu().numpy()
     assert rel_max(got, want16) <= TOL and rel_l1(got, want16) <= TOL
-    # one 64x64 tile per CU at most: the launcher splits the positions over two groups of waves, or over four on
-    # 32-row tiles where those fit the CUs as well (config 4b)
-    tiles = (M + 63) // 64 * ((K + 63) // 64)
-    if (M + 31) // 32 * ((K + 63) // 64) <= cus and C >= 256:
-        assert L.swc_winograd2x2_conv_last_kernel() == b"stored-split4"
-    elif tiles <= cus:
-        assert L.swc_winograd2x2_conv_last_kernel() == b"stored-split"
+    # one tile per CU at most: the launcher splits the positions over two groups of waves (config 4a), or over four
+    # on 32-row tiles where those fit the CUs as well (config 4b)
+    props = torch.cuda.get_device_properties(dev)
+    assert L.swc_winograd2x2_conv_last_kernel().decode() in expected_stored_launch(M, C, K, cus, props.L2_cache_size)

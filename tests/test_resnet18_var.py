@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import rel_max
+from helpers import expected_stored_launch, rel_max
 
 
 def test_topology_matches_reference_graph():
@@ -180,16 +180,7 @@ def test_layers_at_batch_128(oracle, hw, C, K, precision):
     if precision == "fp32":
         assert kernel != "sync", kernel   # every model shape runs on one of the copy-ring tilings
     if stored:
-        # The launcher reads the CU count and the L2 size from the device; so does the expectation.  More 64x64
-        # tiles than CUs at every layer of an MI355X; weights that fill an L2 (4 MiB there) take the deeper ring.
+        # The launcher reads the CU count and the L2 size from the device; so does the expectation.
         props = torch.cuda.get_device_properties(dev)
         M = N * ((hw + 1) // 2) ** 2
-        tiles = -(-M // 64) * -(-K // 64)
-        if C in (128, 256, 512) and K % 64 == 0 and -(-M // 128) * (K // 64) * 4 >= 3 * props.multi_processor_count:
-            assert kernel == "stored-tall", kernel      # enough 128-row x 64-column tiles to go round
-        elif -(-M // 32) * -(-K // 64) <= props.multi_processor_count and C >= 256:
-            assert kernel == "stored-split4", kernel
-        elif tiles <= props.multi_processor_count:
-            assert kernel == "stored-split", kernel
-        else:
-            assert kernel == ("stored-ring4" if 16 * C * K * 2 >= props.L2_cache_size else "stored-ring3"), kernel
+        assert kernel in expected_stored_launch(M, C, K, props.multi_processor_count, props.L2_cache_size), kernel
