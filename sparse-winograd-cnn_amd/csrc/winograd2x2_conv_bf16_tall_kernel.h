@@ -29,7 +29,7 @@ __device__ __forceinline__ void lds_copy_run4(unsigned v0, unsigned v1, unsigned
     static_assert(OFF >= 0 && OFF + 3 * 1024 < 4096, "13-bit immediate offset");
     asm volatile(
         "s_add_i32 m0, %5, %6\n\t"
-        "s_nop 0\n\t"
+        "s_nop 3\n\t"
         "global_load_lds_dwordx4 %0, %4 offset:%7\n\t"
         "global_load_lds_dwordx4 %1, %4 offset:%8\n\t"
         "global_load_lds_dwordx4 %2, %4 offset:%9\n\t"
@@ -45,7 +45,7 @@ __device__ __forceinline__ void lds_copy_run2(unsigned v0, unsigned v1, const ch
     static_assert(OFF >= 0 && OFF + 1024 < 4096, "13-bit immediate offset");
     asm volatile(
         "s_add_i32 m0, %3, %4\n\t"
-        "s_nop 0\n\t"
+        "s_nop 3\n\t"
         "global_load_lds_dwordx4 %0, %2 offset:%5\n\t"
         "global_load_lds_dwordx4 %1, %2 offset:%6"
         :

@@ -465,6 +465,10 @@ __device__ __forceinline__ void async_copy16(const float *base, unsigned voff, u
 {
     // The "s" constraints need values the compiler has in scalar registers; under register pressure
     // it sometimes computes uniform values on the vector unit, so pin them (a no-op when already scalar).
+    // When it is not a no-op, the v_readfirstlane lands right in front of this statement, and a memory
+    // instruction may read a scalar register only five cycles after a vector instruction wrote it; the
+    // compiler cannot check that inside an assembly statement, so the statement keeps the distance itself
+    // (s_mov + s_nop 3; one cycle of it is what the load needs behind the write of M0 anyway).
     const size_t b = reinterpret_cast<size_t>(base);
     const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(b));
     const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(b >> 32));
@@ -472,7 +476,7 @@ __device__ __forceinline__ void async_copy16(const float *base, unsigned voff, u
     lds_base = __builtin_amdgcn_readfirstlane(lds_base);
     asm volatile(
         "s_mov_b32 m0, %2\n\t"
-        "s_nop 0\n\t"
+        "s_nop 3\n\t"
         "global_load_lds_dwordx4 %0, %1"
         :
         : "v"(voff), "s"(base), "s"(lds_base)

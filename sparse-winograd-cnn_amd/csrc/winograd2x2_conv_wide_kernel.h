@@ -113,7 +113,7 @@ __device__ __forceinline__ void async_copy16_imm(const float *base, unsigned vof
     lds_base = __builtin_amdgcn_readfirstlane(lds_base);
     asm volatile(
         "s_add_i32 m0, %2, %3\n\t"
-        "s_nop 0\n\t"
+        "s_nop 3\n\t"
         "global_load_lds_dwordx4 %0, %1"
         :
         : "v"(voff), "s"(base), "s"(lds_base), "n"(LDS_IMM)

@@ -38,7 +38,7 @@ __device__ __forceinline__ void lds_copy_pair(unsigned v0, unsigned v1, const fl
 {
     asm volatile(
         "s_add_i32 m0, %3, %4\n\t"
-        "s_nop 0\n\t"
+        "s_nop 3\n\t"
         "global_load_lds_dwordx4 %0, %2\n\t"
         "global_load_lds_dwordx4 %1, %2 offset:1024"
         :
@@ -50,7 +50,7 @@ __device__ __forceinline__ void lds_copy_quad(unsigned v0, unsigned v1, unsigned
 {
     asm volatile(
         "s_add_i32 m0, %5, %6\n\t"
-        "s_nop 0\n\t"
+        "s_nop 3\n\t"
         "global_load_lds_dwordx4 %0, %4\n\t"
         "global_load_lds_dwordx4 %1, %4 offset:1024\n\t"
         "global_load_lds_dwordx4 %2, %4 offset:2048\n\t"
