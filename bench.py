@@ -231,7 +231,7 @@ SWEEP_SHAPES = [(("N%d %dx%d %d->%d" % (n, hw, hw, c, k)), n, hw, c, k)
     ("N4 56x56 256->64", 4, 56, 256, 64), ("N100 10x10 320->160", 100, 10, 320, 160),
     ("N24 28x28 96->192", 24, 28, 96, 192), ("N12 14x14 1024->256", 12, 14, 1024, 256), ("N200 8x8 64->320", 200, 8, 64, 320),
     ("N2 224x224 32->64", 2, 224, 32, 64), ("N64 12x12 384->384", 64, 12, 384, 384)]
-TILINGS = ("ring32", "ring16", "tall16", "short16", "wide48")
+TILINGS = ("ring32", "ring16", "tall16", "short16", "wide48", "wide48x64")
 
 
 def bench_sweep(args, torch, dev):

@@ -44,7 +44,8 @@ SWC_API const char *swc_version(void);
  * thread's last swc_winograd2x2_conv / _conv_bf16 / _conv_epilogue / _conv_bf16in call launched ("" before the
  * first): "sync" (any shape and alignment), "ring32" / "ring16" (64x64 tiles, 32- / 16-channel steps),
  * "tall16" / "short16" (row groups of up to 112 / 32 rows, dealt evenly over the CUs), "wide48" (48 rows x 128
- * columns per workgroup, left-over rows as extra tiles split along the channels; C % 64 == 0, K % 128 == 0); for
+ * columns per workgroup, left-over rows as extra tiles split along the channels; C % 64 == 0, K % 128 == 0),
+ * "wide48x64" (the same with 64 columns per workgroup; K % 64 == 0); for
  * bf16-stored operands "stored-ring3" / "stored-ring4" (64x64 tiles, 3- / 4-deep copy ring) / "stored-split"
  * (small grids: the 16 positions of a tile split over two groups of waves, whose partial sums are added at the
  * end) / "stored-split4" (smaller grids still: 32-row tiles, four groups of waves) / "stored-tall" (128x64
@@ -55,8 +56,8 @@ SWC_API const char *swc_version(void);
 SWC_API const char *swc_winograd2x2_conv_last_kernel(void);
 /* Diagnostic with no counterpart in the reference, for benchmarks and tests that compare the tilings: makes
  * the calling thread's later swc_winograd2x2_conv calls
- * use the named kernel ("ring32", "ring16", "tall16", "short16", "wide48", "sync") where the shapes allow it and
- * "sync" where they do not; NULL or "" gives the choice back to the launcher.  The data gradient of
+ * use the named kernel ("ring32", "ring16", "tall16", "short16", "wide48", "wide48x64", "sync") where the shapes
+ * allow it and "sync" where they do not; NULL or "" gives the choice back to the launcher.  The data gradient of
  * swc_winograd2x2_conv_grad follows it too: "wide48" takes its wide-tile kernel where the shapes allow it, any
  * other name its position-pair kernel.  Returns SWC_ERR_UNSUPPORTED for an unknown name. */
 SWC_API int swc_winograd2x2_conv_force_tiling(const char *name);

@@ -47,7 +47,7 @@ extern "C" int swc_winograd2x2_conv_force_tiling(const char *name)
         swc::g_forced_tiling[0] = '\0';
         return SWC_OK;
     }
-    for (const char *known : {"sync", "ring32", "ring16", "tall16", "short16", "wide48"}) {
+    for (const char *known : {"sync", "ring32", "ring16", "tall16", "short16", "wide48", "wide48x64"}) {
         if (std::strcmp(name, known) == 0) {
             std::strcpy(swc::g_forced_tiling, known);
             return SWC_OK;

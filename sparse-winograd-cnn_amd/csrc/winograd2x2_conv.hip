@@ -79,6 +79,7 @@ int conv_entry(const float *Input, const float *Weight, float *Output, int C, in
     note_conv_kernel(tiling_name(pick.tiling));
     switch (pick.tiling) {
         case TILING_WIDE48:
+        case TILING_WIDE48X64:
             return launch_wide48(Input, Weight, Output, M, C, K, nW, pick.wide, ep.scale, ep.shift, ep.residual, ep.residual_relu, s);
         case TILING_TALL16:
             return launch_async<Tall, 2, false>(Input, Weight, Output, M, C, K, nH, nW, pick.rows_per_wg, ep, s);

@@ -45,25 +45,30 @@ inline size_t device_l2_bytes()
 struct WidePlan {
     bool ok = false;
     bool extra = false;
+    int bn = 128;   // columns per workgroup: 128 (wave tile 48x32) or 64 (48x16)
     size_t groups = 0, rows_per_wg = 0, main_rows = 0, wgs = 0;
     double units = 0;
 };
 
-// The kernel takes C in pairs of 32-channel steps, whole 128-column groups, 16-byte granules, 32-bit byte offsets
-// into the activations of one position and 31-bit ones into the output.
-inline bool wide48_eligible(const void *A, const void *B, size_t M, int R, int N)
+// The kernel takes C in pairs of 32-channel steps, whole column groups of bn = 128 or 64, 16-byte granules, 32-bit
+// byte offsets into the activations of one position and 31-bit ones into the output.
+inline bool wide48_eligible(const void *A, const void *B, size_t M, int R, int N, int bn = 128)
 {
-    return R % 64 == 0 && N % 128 == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0 &&
+    return R % 64 == 0 && N % bn == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0 &&
            M >= 48 && M * static_cast<size_t>(R) * 4 < (1ull << 32) && M * 16 * static_cast<size_t>(N) < (1ull << 31) &&
            static_cast<size_t>(R) * N * 16 * 4 < (1ull << 40);
 }
 
-// Either full 48-row groups in whole passes over the chip with the rest as extra tiles (6.25 units per pass), or
-// the rows levelled over as many groups as fill whole passes (6 units), whichever makes fewer units in total.
-inline WidePlan plan_wide48(size_t M, int N, size_t cus)
+// Either full 48-row groups in whole passes over the chip with the rest as extra tiles (6.25 units per pass with
+// 128-column workgroups, 3.25 with 64-column ones), or the rows levelled over as many groups as fill whole passes
+// (6 or 3 units), whichever makes fewer units in total.
+inline WidePlan plan_wide48(size_t M, int N, size_t cus, int bn = 128)
 {
     WidePlan best;
-    const size_t tiles_n = static_cast<size_t>(N) / 128;
+    best.bn = bn;
+    const size_t tiles_n = static_cast<size_t>(N) / bn;
+    const double unit = bn == 128 ? 6.0 : 3.0;
+    const size_t xct = static_cast<size_t>(bn) / 16;   // extra tiles per left-over row tile and column group
     if (tiles_n == 0 || M < 48) return best;
     auto passes_of = [&](size_t wgs) { return static_cast<double>((wgs + cus - 1) / cus); };
     {   // levelled
@@ -78,7 +83,7 @@ inline WidePlan plan_wide48(size_t M, int N, size_t cus)
         best.rows_per_wg = rows;
         best.main_rows = M;
         best.wgs = groups * tiles_n;
-        best.units = passes_of(best.wgs) * 6.0;
+        best.units = passes_of(best.wgs) * unit;
     }
     {   // full groups plus extra tiles
         const size_t gfull = M / 48;
@@ -86,8 +91,8 @@ inline WidePlan plan_wide48(size_t M, int N, size_t cus)
         if (groups == 0) groups = gfull;
         const size_t main_rows = groups * 48;
         const size_t left_tiles = (M - main_rows + 15) / 16;
-        if (left_tiles > 0 && left_tiles * 8 <= groups) {
-            const double units = passes_of(groups * tiles_n) * 6.25;
+        if (left_tiles > 0 && left_tiles * xct <= groups) {
+            const double units = passes_of(groups * tiles_n) * (unit + 0.25);
             if (units < best.units) {
                 best.extra = true;
                 best.groups = groups;
@@ -107,7 +112,10 @@ int launch_bf16_tall(const unsigned short *TI16, const unsigned short *Wt16, flo
                      size_t rows_per_wg, const float *scale, const float *shift, const float *residual, int residual_relu,
                      hipStream_t stream);
 
-// Defined in winograd2x2_conv_wide.hip.
+// Defined in winograd2x2_conv_wide.hip (128-column workgroups) and winograd2x2_conv_wide64.hip (64-column ones);
+// launch_wide48 hands a plan with bn == 64 on to the second.
+int launch_wide48_n64(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nW, const WidePlan &plan,
+                      const float *scale, const float *shift, const float *residual, int residual_relu, hipStream_t stream);
 int launch_wide48(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nW, const WidePlan &plan,
                   const float *scale, const float *shift, const float *residual, int residual_relu, hipStream_t stream);
 
@@ -122,7 +130,7 @@ using Tile16 = ConvCfg<64, 64, 16, 2, 2>;
 using Tall = ConvCfg<112, 64, 32, 1, 4, 2, 16>;
 using Short = ConvCfg<32, 64, 64, 1, 4, 3, 16>;
 
-enum Tiling { TILING_SYNC = 0, TILING_RING32, TILING_RING16, TILING_TALL16, TILING_SHORT16, TILING_WIDE48 };
+enum Tiling { TILING_SYNC = 0, TILING_RING32, TILING_RING16, TILING_TALL16, TILING_SHORT16, TILING_WIDE48, TILING_WIDE48X64 };
 inline const char *tiling_name(Tiling t)
 {
     switch (t) {
@@ -131,6 +139,7 @@ inline const char *tiling_name(Tiling t)
         case TILING_TALL16: return "tall16";
         case TILING_SHORT16: return "short16";
         case TILING_WIDE48: return "wide48";
+        case TILING_WIDE48X64: return "wide48x64";
         default: return "sync";
     }
 }
@@ -195,9 +204,13 @@ inline TilingChoice choose_tiling(const void *A, const void *B, size_t M, int R,
     // wide48 (forward only): 48-row x 128-column workgroups, left-over rows dealt out as extra tiles.
     const bool ok_wide = forward && wide48_eligible(A, B, M, R, N);
     const WidePlan wide = ok_wide ? plan_wide48(M, N, cus) : WidePlan();
+    // the same with 64-column workgroups (wave tile 48x16: more LDS reads per MFMA, twice the workgroups)
+    const bool ok_wide64 = forward && wide48_eligible(A, B, M, R, N, 64);
+    const WidePlan wide64 = ok_wide64 ? plan_wide48(M, N, cus, 64) : WidePlan();
     if (const char *f = forced_conv_tiling()) {
         const std::string_view want(f);
         if (want == "wide48" && wide.ok) return {TILING_WIDE48, wide.rows_per_wg, wide};
+        if (want == "wide48x64" && wide64.ok) return {TILING_WIDE48X64, wide64.rows_per_wg, wide64};
         if (want == "ring32" && ok32) return {TILING_RING32, Tile32::BM};
         if (want == "ring16" && ok16) return {TILING_RING16, Tile16::BM};
         if (want == "tall16" && ok_tall) return {TILING_TALL16, rows_tall};
@@ -213,6 +226,15 @@ inline TilingChoice choose_tiling(const void *A, const void *B, size_t M, int R,
     const double cost_short = ok_short ? passes(wgs_short, cus) * 2.0 * w_short : 1e30;
     // wide48: a unit of its work measured 9 % more than ring32's with one workgroup per CU, 1 % more with two.
     const double cost_wide = wide.ok ? wide.units * (wide.wgs > cus ? 1.01 : 1.09) : 1e30;
+    // 64-column workgroups: 12 % more per unit (14x14x256 at batch 64: 64 us against 74 for short16; 28x28x128: 62
+    // against 59 for the 128-column workgroups); with 64 channels a position is two steps and the output transform's
+    // share grows (56x56x64 at batch 64, four workgroups per CU: level with tall16; at batch 16, one per CU: 20 us
+    // against 22 for short16), so with fewer than 128 channels only for a single pass, and never for less than a full
+    // pass of workgroups.
+    const double cost_wide64 =
+        wide64.ok && (R >= 128 || wide64.wgs <= cus) && wide64.wgs >= cus ? wide64.units * 1.12 : 1e30;
+    if (cost_wide64 < cost_wide && cost_wide64 < cost32 && cost_wide64 < cost_tall && cost_wide64 < cost_short)
+        return {TILING_WIDE48X64, wide64.rows_per_wg, wide64};
     if (wide.ok && cost_wide < cost32 && cost_wide < cost_tall && cost_wide < cost_short) return {TILING_WIDE48, wide.rows_per_wg, wide};
     if (ok_tall && cost_tall < cost32 && cost_tall <= cost_short) return {TILING_TALL16, rows_tall};
     if (ok_short && cost_short < cost32) return {TILING_SHORT16, rows_short};

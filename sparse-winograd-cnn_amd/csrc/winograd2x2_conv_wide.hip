@@ -26,7 +26,8 @@ int launch_wide48_as(const float *TI, const float *Wt, float *Out, size_t M, int
 int launch_wide48(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nW, const WidePlan &plan,
                   const float *scale, const float *shift, const float *residual, int residual_relu, hipStream_t stream)
 {
-    if (!plan.ok || !wide48_eligible(TI, Wt, M, C, K) || plan.groups * (K / 128) >= (1ull << 31)) return SWC_ERR_UNSUPPORTED;
+    if (!plan.ok || !wide48_eligible(TI, Wt, M, C, K, plan.bn) || plan.groups * (K / plan.bn) >= (1ull << 31)) return SWC_ERR_UNSUPPORTED;
+    if (plan.bn == 64) return launch_wide48_n64(TI, Wt, Out, M, C, K, nW, plan, scale, shift, residual, residual_relu, stream);
     ConvEpilogue ep;
     ep.scale = scale;
     ep.shift = shift;

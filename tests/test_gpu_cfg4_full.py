@@ -42,8 +42,11 @@ def test_config4_full_size(oracle, layer):
     got = winograd2x2_conv(ti, gpu(w, dev)).cpu().numpy()
     assert got.shape == want.shape == (N, 2 * nT, 2 * nT, K)
     assert rel_max(got, want) <= TOL and rel_l1(got, want) <= TOL
-    if cus == 256:   # the tiling follows from the CU count: 32-row groups fill an MI355X where 64-row tiles leave CUs idle
-        assert L.swc_winograd2x2_conv_last_kernel() == b"short16"
+    if cus == 256:
+        # the tiling follows from the CU count: on an MI355X 32-row groups fill the device at config 4b where 64-row
+        # tiles leave CUs idle; at config 4a one 48-row x 64-column workgroup per CU does (64 of them carry one of the
+        # 16 tiles of the 64 left-over rows)
+        assert L.swc_winograd2x2_conv_last_kernel() == (b"wide48x64" if name == "4a" else b"short16")
 
     # bf16 operands, fp32 planes: against the oracle fed the same rounded operands
     want16 = oracle.conv(oracle.round_bf16(ti_want), oracle.round_bf16(w), acc64=True)

@@ -138,11 +138,15 @@ def test_conv_shapes_reach_every_kernel(dev):
     import swc_hip
     _, conv = ops()
     seen = set()
-    for shape in CONV_SHAPES + [(64, 14, 14, 128, 128)]:   # the last one: benchmark config 3, checked in full below
+    # the last two: benchmark config 3, checked in full below, and config 4a's geometry (one 48-row x 64-column
+    # workgroup per CU of an MI355X), checked in full in test_gpu_cfg4_full.py
+    for shape in CONV_SHAPES + [(64, 14, 14, 128, 128), (64, 7, 7, 256, 256)]:
         B, nH, nW, C, K = shape
         conv(torch.zeros((16, B, nH, nW, C), device=dev), torch.zeros((16, C, K), device=dev))
         seen.add(swc_hip.lib().swc_winograd2x2_conv_last_kernel().decode())
-    assert seen == {"sync", "ring32", "ring16", "tall16", "short16", "wide48"}, seen
+    assert seen >= {"sync", "ring32", "ring16", "tall16", "short16", "wide48"}, seen
+    if torch.cuda.get_device_properties(dev).multi_processor_count == 256:
+        assert "wide48x64" in seen, seen
 
 
 @pytest.mark.parametrize("tiling", ["ring32", "ring16", "tall16", "short16", "sync"])
@@ -180,9 +184,19 @@ WIDE48_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("shape", WIDE48_SHAPES)
-def test_conv_fp32_wide48(oracle, dev, shape):
-    """The wide48 tiling forced on shapes below the size at which the launcher picks it by itself.  Its output
+# The same kernel with 64-column workgroups ("wide48x64") takes K % 64 == 0.
+WIDE48X64_SHAPES = [
+    (8, 14, 14, 128, 64),    # one column group, levelled
+    (3, 5, 7, 64, 192),      # three column groups, levelled: M = 105
+    (2, 20, 20, 64, 64),     # 16 full groups + 2 extra row tiles of 4 tiles each
+    (2, 2, 197, 128, 128),   # two column groups, the second extra row tile holds 4 rows
+    (16, 7, 7, 256, 256),    # config 4a's geometry at a quarter of its batch
+]
+
+
+@pytest.mark.parametrize("shape,tiling", [(s, "wide48") for s in WIDE48_SHAPES] + [(s, "wide48x64") for s in WIDE48X64_SHAPES])
+def test_conv_fp32_wide48(oracle, dev, shape, tiling):
+    """The wide48 tilings forced on shapes below the size at which the launcher picks them by itself.  Their output
     transform is taken in another association than the reference's (sum/difference pairs, partial sums continued
     by the matrix pipes), so besides the tolerance check the integer check pins every sign and the scatter exactly."""
     import swc_hip
@@ -196,10 +210,10 @@ def test_conv_fp32_wide48(oracle, dev, shape):
     scale = (0.5 + rng.random(K)).astype(np.float32) * rng.choice([-1, 1], K).astype(np.float32)
     shift = rng.standard_normal(K).astype(np.float32)
     res = rng.standard_normal((B, 2 * nH, 2 * nW, K)).astype(np.float32)
-    assert L.swc_winograd2x2_conv_force_tiling(b"wide48") == 0
+    assert L.swc_winograd2x2_conv_force_tiling(tiling.encode()) == 0
     try:
         got = conv(gpu(ti, dev), gpu(w, dev))
-        assert L.swc_winograd2x2_conv_last_kernel().decode() == "wide48"
+        assert L.swc_winograd2x2_conv_last_kernel().decode() == tiling
         got_int = conv(gpu(ti_int, dev), gpu(w_int, dev)).cpu().numpy()
         got_ep = conv(gpu(ti, dev), gpu(w, dev), scale=gpu(scale, dev), shift=gpu(shift, dev), residual=gpu(res, dev),
                       residual_relu=True).cpu().numpy()
