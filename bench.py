@@ -37,8 +37,8 @@ MEASURED_TRAFFIC = {
     ("cfg3", "fp32", "imtrans"): (None, (12575.0 * 2 + 100422.5) * 1024),         # algorithmic 128.45 MB
     ("cfg2", "fp32", "conv"): ("tall16", (108090.0 * 2 + 50176.0) * 1024),       # algorithmic 257.2 MB
     ("cfg2", "fp32", "imtrans"): (None, (25126.2 * 2 + 200811.9) * 1024),
-    ("cfg4a", "fp32", "conv"): ("wide48x64", (42442.5 * 2 + 12544.0) * 1024),    # algorithmic 68.4 MB
-    ("cfg4a", "fp32", "imtrans"): (None, (6433.6 * 2 + 50176.0) * 1024),
+    ("cfg4a", "fp32", "conv"): ("wide48x64", (43381.5 * 2 + 12544.0) * 1024),    # algorithmic 68.4 MB
+    ("cfg4a", "fp32", "imtrans"): (None, (6431.2 * 2 + 50176.0) * 1024),
     ("cfg4b", "fp32", "conv"): ("short16", (83452.0 * 2 + 8192.0) * 1024),       # algorithmic 58.7 MB
     ("cfg4b", "fp32", "imtrans"): (None, (3175.0 * 2 + 32768.0) * 1024),
     ("cfg3", "bf16_stored", "conv"): ("stored-tall", (30373.5 * 2 + 25088.0) * 1024),    # algorithmic 77.6 MB

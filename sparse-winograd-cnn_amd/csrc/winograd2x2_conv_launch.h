@@ -112,10 +112,13 @@ int launch_bf16_tall(const unsigned short *TI16, const unsigned short *Wt16, flo
                      size_t rows_per_wg, const float *scale, const float *shift, const float *residual, int residual_relu,
                      hipStream_t stream);
 
-// Defined in winograd2x2_conv_wide.hip (128-column workgroups) and winograd2x2_conv_wide64.hip (64-column ones);
+// Defined in winograd2x2_conv_wide.hip (128-column workgroups) and winograd2x2_conv_wide64*.hip (64-column ones);
 // launch_wide48 hands a plan with bn == 64 on to the second.
 int launch_wide48_n64(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nW, const WidePlan &plan,
                       const float *scale, const float *shift, const float *residual, int residual_relu, hipStream_t stream);
+int launch_wide48_n64_ring4(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nW, const WidePlan &plan,
+                            const float *scale, const float *shift, const float *residual, int residual_relu,
+                            hipStream_t stream);
 int launch_wide48(const float *TI, const float *Wt, float *Out, size_t M, int C, int K, int nW, const WidePlan &plan,
                   const float *scale, const float *shift, const float *residual, int residual_relu, hipStream_t stream);
 
@@ -226,11 +229,12 @@ inline TilingChoice choose_tiling(const void *A, const void *B, size_t M, int R,
     const double cost_short = ok_short ? passes(wgs_short, cus) * 2.0 * w_short : 1e30;
     // wide48: a unit of its work measured 9 % more than ring32's with one workgroup per CU, 1 % more with two.
     const double cost_wide = wide.ok ? wide.units * (wide.wgs > cus ? 1.01 : 1.09) : 1e30;
-    // 64-column workgroups: 12 % more per unit (14x14x256 at batch 64: 64 us against 74 for short16; 28x28x128: 62
-    // against 59 for the 128-column workgroups); with 64 channels a position is two steps and the output transform's
-    // share grows (56x56x64 at batch 64, four workgroups per CU: level with tall16; at batch 16, one per CU: 20 us
-    // against 22 for short16), so with fewer than 128 channels only for a single pass, and never for less than a full
-    // pass of workgroups.
+    // 64-column workgroups: 12 % more per unit (14x14x256 at batch 64: 57 us against 70 for short16; 28x28x128: 56
+    // against 54 for the 128-column workgroups).  With 64 channels a position is two steps, the ring has two slots
+    // and the output transform's share grows: at 56x56x64, batch 64 (four workgroups per CU) the kernel alone is 4 %
+    // faster than tall16 on cache-resident planes, but the transform + convolution pair, whose planes come from
+    // HBM, is 4 % slower (110 us against 106); at batch 16 (one workgroup per CU) it wins both ways (20 us against
+    // 22 for short16).  So below 128 channels only for a single pass, and never for less than a full pass.
     const double cost_wide64 =
         wide64.ok && (R >= 128 || wide64.wgs <= cus) && wide64.wgs >= cus ? wide64.units * 1.12 : 1e30;
     if (cost_wide64 < cost_wide && cost_wide64 < cost32 && cost_wide64 < cost_tall && cost_wide64 < cost_short)

@@ -1,6 +1,6 @@
 // Launches of the wide48 kernel (winograd2x2_conv_wide_kernel.h) with 64-column workgroups (wave tile 48x16), for
 // shapes where 128-column workgroups are too few to fill the device.  A translation unit of its own: its four
-// instantiations take minutes to compile.  Part of what stands in for Winograd2x2ConvComputeLauncher
+// instantiations take minutes to compile (the four with a 4-slot ring are in winograd2x2_conv_wide64_ring4.hip).  Part of what stands in for Winograd2x2ConvComputeLauncher
 // (winograd2x2_cublas/winograd2x2_conv/winograd2x2_conv_cuda.cu.cc:65-93).
 #include "winograd2x2_conv_wide_kernel.h"
 #include "winograd2x2_conv_launch.h"
@@ -27,6 +27,9 @@ int launch_wide48_n64(const float *TI, const float *Wt, float *Out, size_t M, in
                       const float *scale, const float *shift, const float *residual, int residual_relu, hipStream_t stream)
 {
     if (!plan.ok || plan.bn != 64 || !wide48_eligible(TI, Wt, M, C, K, 64)) return SWC_ERR_UNSUPPORTED;
+    // With whole rounds of four steps per position the copies run three steps ahead (14x14x256 at batch 64 over
+    // buffers that are not cache-resident: 65 us against 76).
+    if (C % 128 == 0) return launch_wide48_n64_ring4(TI, Wt, Out, M, C, K, nW, plan, scale, shift, residual, residual_relu, stream);
     ConvEpilogue ep;
     ep.scale = scale;
     ep.shift = shift;

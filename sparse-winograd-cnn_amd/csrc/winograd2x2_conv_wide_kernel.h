@@ -70,10 +70,12 @@ constexpr unsigned long long wide_pos_packed()
 
 // BK channels per step; TN 16-column tiles per wave (the workgroup's tile is 48 rows x 64*TN columns);
 // EXTRA: the workgroup also carries a 16x16 tile of the left-over rows; OCC waves per SIMD; EPI: the stores apply
-// scale/shift and add a residual (ConvEpilogue).  The ring has two slots.
-template <int BK_, int TN_, bool EXTRA_, int OCC_, bool EPI_>
+// scale/shift and add a residual (ConvEpilogue).  The ring has NSTAGE slots: two, or four for grids of one workgroup
+// per CU, where nothing else hides the latency of a tile that comes from HBM (the copies then run three steps
+// ahead instead of one); a position's steps go round the slots a whole number of times, so C % (NSTAGE*BK) == 0.
+template <int BK_, int TN_, bool EXTRA_, int OCC_, bool EPI_, int NSTAGE_ = 2>
 struct WideCfg {
-    static constexpr int BK = BK_, TN = TN_, OCC = OCC_, NSTAGE = 2;
+    static constexpr int BK = BK_, TN = TN_, OCC = OCC_, NSTAGE = NSTAGE_;
     static constexpr bool EXTRA = EXTRA_, EPI = EPI_;
     static constexpr int TM = 3, NT = 256, BM = 16 * TM, BN = 64 * TN;
     static constexpr int AROWS = BM + (EXTRA ? 16 : 0);   // rows of the A tile in LDS
@@ -93,6 +95,8 @@ struct WideCfg {
     static constexpr int PLANE_OPS = TM * TN * 4;         // store instructions of one output plane
     static constexpr bool EARLY = !EPI;                   // planes are stored as they become final (a residual is read at the end instead)
     static_assert(BK == 32 || BK == 64, "a step is two or four operand groups");
+    static_assert(NSTAGE == 2 || NSTAGE == 4, "two or four ring slots");
+    static_assert(LDS_BYTES <= 160 * 1024, "fits a CU");
     static_assert(TN == 1 || TN == 2, "64 or 128 columns");
     static_assert(NBW % 4 == 0, "every wave issues the same number of B copies");
     static_assert(STAGE_BYTES % 256 == 0, "operand reads address a slot through their immediate offsets");
@@ -224,15 +228,29 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
         float4 a[KH][TM];
         float b[KH][4][TN];
     };
-    unsigned a_lane[KS];  // A: row li of tile 0, the lane's chunk of group k8
-#pragma unroll
-    for (int k8 = 0; k8 < KS; ++k8) a_lane[k8] = (li * CH + ((4 * k8 + lg) ^ (li % CH))) * 16u;
+    // An LDS read addresses base register + 16-bit immediate: a ring of more than 64 KiB is read through two sets of
+    // lane bases, one per half of the ring (NBANK == 2), so that slot, tile and group stay in the immediate.
+    constexpr int NBANK = W::LDS_BYTES > 65536 ? 2 : 1, BANK_STAGES = W::NSTAGE / NBANK;
+    unsigned a_lane[NBANK][KS];  // A: row li of tile 0, the lane's chunk of group k8
+    unsigned b_lane[NBANK], xa_lane[NBANK], xb_lane[NBANK];
     // B row k sits at k*BN*4 + (k/4)*64 bytes; this lane's rows of group k8 are 16*k8 + 4*lg + t.
-    const unsigned b_lane = A_BYTES + 4u * lg * (BN * 4) + lg * 64u + wcol * 4u;
     // Extra tile: this wave's channels of a step are XK*wave + XM*lg + t, t < XM.
     const int x_ch = XK * wave + XM * lg;
-    const unsigned xa_lane = (W::BM + li) * (BK * 4) + (((x_ch / 4) ^ (li % CH)) * 16u) + (x_ch % 4) * 4u;
-    const unsigned xb_lane = A_BYTES + x_ch * (BN * 4) + (x_ch / 4) * 64u + (xc * 16u + li) * 4u;
+#pragma unroll
+    for (int bk = 0; bk < NBANK; ++bk) {
+        const unsigned at = bk * BANK_STAGES * STAGE_BYTES;
+#pragma unroll
+        for (int k8 = 0; k8 < KS; ++k8) a_lane[bk][k8] = at + (li * CH + ((4 * k8 + lg) ^ (li % CH))) * 16u;
+        b_lane[bk] = at + A_BYTES + 4u * lg * (BN * 4) + lg * 64u + wcol * 4u;
+        xa_lane[bk] = at + (W::BM + li) * (BK * 4) + (((x_ch / 4) ^ (li % CH)) * 16u) + (x_ch % 4) * 4u;
+        xb_lane[bk] = at + A_BYTES + x_ch * (BN * 4) + (x_ch / 4) * 64u + (xc * 16u + li) * 4u;
+        if (bk > 0) {
+            // kept in registers of their own (the compiler would otherwise fold them back into base + constant)
+#pragma unroll
+            for (int k8 = 0; k8 < KS; ++k8) asm volatile("" : "+v"(a_lane[bk][k8]));
+            asm volatile("" : "+v"(b_lane[bk]), "+v"(xa_lane[bk]), "+v"(xb_lane[bk]));
+        }
+    }
     struct ExtraFrag {
         float a[XM], b[XM];
     };
@@ -240,28 +258,30 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
     constexpr int NUB = 2 * TN, NU = KH * (TM + NUB);
     auto lds_f32 = [&](unsigned byte) __attribute__((always_inline)) { return *reinterpret_cast<const float *>(wsmem + byte); };
     auto read_unit = [&](HalfFrag &F, auto stage_tag, int h, int u) __attribute__((always_inline)) {
-        constexpr unsigned st = decltype(stage_tag)::value * STAGE_BYTES;
+        constexpr int bank = decltype(stage_tag)::value / BANK_STAGES;
+        constexpr unsigned st = (decltype(stage_tag)::value % BANK_STAGES) * STAGE_BYTES;
         const int k8l = u / (TM + NUB), v = u % (TM + NUB);
         const int k8 = h * KH + k8l;
         if (v < TM) {
-            F.a[k8l][v] = *reinterpret_cast<const float4 *>(wsmem + a_lane[k8] + (st + v * 16 * BK * 4));
+            F.a[k8l][v] = *reinterpret_cast<const float4 *>(wsmem + a_lane[bank][k8] + (st + v * 16 * BK * 4));
         } else {
             const int tn = (v - TM) / 2, tp = (v - TM) % 2;
             const unsigned at = st + (16 * k8 + 2 * tp) * (BN * 4) + 4 * k8 * 64 + tn * 256;
-            F.b[k8l][2 * tp][tn] = lds_f32(b_lane + at);
-            F.b[k8l][2 * tp + 1][tn] = lds_f32(b_lane + at + BN * 4);
+            F.b[k8l][2 * tp][tn] = lds_f32(b_lane[bank] + at);
+            F.b[k8l][2 * tp + 1][tn] = lds_f32(b_lane[bank] + at + BN * 4);
         }
     };
     constexpr int NXU = EXTRA ? 1 + XM / 2 : 0;
     auto read_extra = [&](ExtraFrag &X, auto stage_tag, int u) __attribute__((always_inline)) {
-        constexpr unsigned st = decltype(stage_tag)::value * STAGE_BYTES;
+        constexpr int bank = decltype(stage_tag)::value / BANK_STAGES;
+        constexpr unsigned st = (decltype(stage_tag)::value % BANK_STAGES) * STAGE_BYTES;
         if (u == 0) {
             if constexpr (XM == 2) {
-                const float2 v = *reinterpret_cast<const float2 *>(wsmem + xa_lane + st);
+                const float2 v = *reinterpret_cast<const float2 *>(wsmem + xa_lane[bank] + st);
                 X.a[0] = v.x;
                 X.a[1] = v.y;
             } else {
-                const float4 v = *reinterpret_cast<const float4 *>(wsmem + xa_lane + st);
+                const float4 v = *reinterpret_cast<const float4 *>(wsmem + xa_lane[bank] + st);
                 X.a[0] = v.x;
                 X.a[1] = v.y;
                 X.a[2 % XM] = v.z;
@@ -269,8 +289,8 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
             }
         } else {
             const int t = 2 * (u - 1);
-            X.b[t] = lds_f32(xb_lane + st + t * (BN * 4));
-            X.b[t + 1] = lds_f32(xb_lane + st + (t + 1) * (BN * 4));
+            X.b[t] = lds_f32(xb_lane[bank] + st + t * (BN * 4));
+            X.b[t + 1] = lds_f32(xb_lane[bank] + st + (t + 1) * (BN * 4));
         }
     };
 
@@ -342,15 +362,14 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
     const float no_residual[4] = {0.f, 0.f, 0.f, 0.f};
 
     using Stage0 = std::integral_constant<int, 0>;
-    using Stage1 = std::integral_constant<int, 1>;
+    constexpr int NSTAGE = W::NSTAGE;
     // ---- prologue: fill the ring, wait for step 0, read its first half -------------------------------------
+    static_for<NSTAGE>([&](auto s_tag) {
 #pragma unroll
-    for (int c = 0; c < LPS; ++c) copy(Stage0{}, c);
-    advance();
-#pragma unroll
-    for (int c = 0; c < LPS; ++c) copy(Stage1{}, c);
-    advance();
-    wait_vmcnt<LPS>();
+        for (int c = 0; c < LPS; ++c) copy(s_tag, c);
+        advance();
+    });
+    wait_vmcnt<(NSTAGE - 1) * LPS>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     HalfFrag F1, F2;
@@ -363,7 +382,7 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
     auto step = [&](auto q_tag, auto first_tag, auto stage_tag) __attribute__((always_inline)) {
         constexpr int q = decltype(q_tag)::value;
         constexpr bool first = decltype(first_tag)::value;
-        using Other = std::integral_constant<int, 1 - decltype(stage_tag)::value>;
+        using Other = std::integral_constant<int, (decltype(stage_tag)::value + 1) % NSTAGE>;   // the next step's slot
         constexpr int dst = kWideDst[q];
         constexpr bool fresh = first && kWideFresh[q];
         constexpr int store_plane = first && W::EARLY ? kWideStoreAt[q] : -1;
@@ -424,9 +443,9 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
             mfma_slot(F2, i, false);
             if (i == 0) {
                 // The tile of the next step is complete once nothing but what was issued after its copies is
-                // outstanding: the stores (and residual loads) of this step's first half.  Memory operations
-                // complete in issue order.
-                constexpr int mine = store_plane >= 0 ? W::PLANE_OPS : 0;
+                // outstanding: the copies of the steps behind it in the ring and the stores (and residual loads)
+                // of this step's first half.  Memory operations complete in issue order.
+                constexpr int mine = (NSTAGE - 2) * LPS + (store_plane >= 0 ? W::PLANE_OPS : 0);
                 wait_vmcnt<(mine < 63 ? mine : 63)>();
                 __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS reads of this step are done
                 __builtin_amdgcn_s_barrier();
@@ -454,14 +473,12 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
         advance();
     };
 
-    // Steps alternate between the two ring slots; a position has an even number of steps, so it starts on slot 0.
+    // Steps go round the ring slots; a position has a multiple of NSTAGE steps, so it starts on slot 0.
     static_for<16>([&](auto q_tag) {
         step(q_tag, std::true_type{}, Stage0{});
-        step(q_tag, std::false_type{}, Stage1{});
-        for (int kc = 2; kc < nkc; kc += 2) {
-            step(q_tag, std::false_type{}, Stage0{});
-            step(q_tag, std::false_type{}, Stage1{});
-        }
+        static_for<NSTAGE - 1>([&](auto s_tag) { step(q_tag, std::false_type{}, std::integral_constant<int, decltype(s_tag)::value + 1>{}); });
+        for (int kc = NSTAGE; kc < nkc; kc += NSTAGE)
+            static_for<NSTAGE>([&](auto s_tag) { step(q_tag, std::false_type{}, s_tag); });
     });
 
     // The surplus copies must have landed before this workgroup's LDS can be handed on.
