@@ -13,9 +13,9 @@ int launch_wide64_as(const float *TI, const float *Wt, float *Out, size_t M, int
                      const ConvEpilogue &ep, hipStream_t stream)
 {
     using W = WideCfg<32, 1, EXTRA, 2, EPI>;
-    static_assert(W::LDS_BYTES <= 64 * 1024, "fits the default dynamic LDS limit");
+    static_assert(W::LAUNCH_LDS_BYTES <= 64 * 1024, "fits the default dynamic LDS limit");
     const unsigned tiles_n = static_cast<unsigned>(K / W::BN);
-    conv_wide48_kernel<W><<<dim3(static_cast<unsigned>(plan.groups) * tiles_n), dim3(W::NT), W::LDS_BYTES, stream>>>(
+    conv_wide48_kernel<W><<<dim3(static_cast<unsigned>(plan.groups) * tiles_n), dim3(W::NT), W::LAUNCH_LDS_BYTES, stream>>>(
         TI, Wt, Out, static_cast<unsigned>(M), C, K, nW, tiles_n, static_cast<unsigned>(plan.rows_per_wg),
         static_cast<unsigned>(plan.main_rows), ep);
     return check_launch();

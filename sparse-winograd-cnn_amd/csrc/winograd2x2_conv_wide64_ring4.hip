@@ -13,12 +13,12 @@ int launch_wide64_ring4_as(const float *TI, const float *Wt, float *Out, size_t 
                      const ConvEpilogue &ep, hipStream_t stream)
 {
     using W = WideCfg<32, 1, EXTRA, 2, EPI, 4>;
-    static_assert(2 * W::LDS_BYTES <= 160 * 1024, "two workgroups per CU");
+    static_assert(2 * W::LAUNCH_LDS_BYTES <= 160 * 1024, "two workgroups per CU");
     struct Tag {};
-    const int st = raise_lds_limit<Tag>(reinterpret_cast<const void *>(conv_wide48_kernel<W>), W::LDS_BYTES);
+    const int st = raise_lds_limit<Tag>(reinterpret_cast<const void *>(conv_wide48_kernel<W>), W::LAUNCH_LDS_BYTES);
     if (st != SWC_OK) return st;
     const unsigned tiles_n = static_cast<unsigned>(K / W::BN);
-    conv_wide48_kernel<W><<<dim3(static_cast<unsigned>(plan.groups) * tiles_n), dim3(W::NT), W::LDS_BYTES, stream>>>(
+    conv_wide48_kernel<W><<<dim3(static_cast<unsigned>(plan.groups) * tiles_n), dim3(W::NT), W::LAUNCH_LDS_BYTES, stream>>>(
         TI, Wt, Out, static_cast<unsigned>(M), C, K, nW, tiles_n, static_cast<unsigned>(plan.rows_per_wg),
         static_cast<unsigned>(plan.main_rows), ep);
     return check_launch();

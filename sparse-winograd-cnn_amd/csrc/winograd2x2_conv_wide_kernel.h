@@ -87,6 +87,12 @@ struct WideCfg {
     static constexpr int B_BYTES = BK * BN * 4 + (BK / 4) * 64;  // 64 bytes after every 4 rows: lane groups read rows 4 apart
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
+    // With two slots a tile is copied one step before its use: less than a trip to HBM takes.  The first step of a
+    // position then also touches the next position's A tiles (one 4-byte global -> LDS load per wave into a landing
+    // area behind the ring that nobody reads), so that their copies find the lines in L2.
+    static constexpr bool TOUCH = NSTAGE == 2;
+    static constexpr int TOUCH_BYTES = TOUCH ? 4 * 256 : 0;
+    static constexpr int LAUNCH_LDS_BYTES = LDS_BYTES + TOUCH_BYTES;
     static constexpr int KS = BK / 16, KH = KS / 2;       // operand groups of 16 channels per step / per half
     static constexpr int NM = KH * 4 * TM * TN;           // MFMAs of a wave's own tiles per half step
     static constexpr int XK = BK / 4, XM = XK / 4;        // extra tile: channels and MFMAs per wave and step
@@ -96,7 +102,8 @@ struct WideCfg {
     static constexpr bool EARLY = !EPI;                   // planes are stored as they become final (a residual is read at the end instead)
     static_assert(BK == 32 || BK == 64, "a step is two or four operand groups");
     static_assert(NSTAGE == 2 || NSTAGE == 4, "two or four ring slots");
-    static_assert(LDS_BYTES <= 160 * 1024, "fits a CU");
+    static_assert(LAUNCH_LDS_BYTES <= 160 * 1024, "fits a CU");
+    static_assert(!TOUCH || BK == 32, "a row of a step's A tile is one 128-byte line");
     static_assert(TN == 1 || TN == 2, "64 or 128 columns");
     static_assert(NBW % 4 == 0, "every wave issues the same number of B copies");
     static_assert(STAGE_BYTES % 256 == 0, "operand reads address a slot through their immediate offsets");
@@ -124,6 +131,23 @@ __device__ __forceinline__ void async_copy16_imm(const float *base, unsigned vof
         : "memory", "scc");
 }
 
+// The same with 4 bytes per lane: what arrives is never read, the point is the lines it pulls into L2.
+__device__ __forceinline__ void async_touch4(const float *base, unsigned voff, unsigned lds_addr)
+{
+    const size_t b = reinterpret_cast<size_t>(base);
+    const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(b));
+    const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(b >> 32));
+    base = reinterpret_cast<const float *>((static_cast<size_t>(hi) << 32) | lo);
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+    asm volatile(
+        "s_mov_b32 m0, %2\n\t"
+        "s_nop 3\n\t"
+        "global_load_lds_dword %0, %1"
+        :
+        : "v"(voff), "s"(base), "s"(lds_addr)
+        : "memory");
+}
+
 // Requirements checked by the launcher: C % (2*BK) == 0, K % BN == 0, TI and Wt 16-byte aligned, M*C*4 < 2^32,
 // the output below 2^31 bytes.  grid.x = groups * tiles_n; the row groups cover main_rows = min(M, groups *
 // rows_per_wg) rows, rows_per_wg <= 48; with EXTRA the rows from main_rows on are the left-over tiles, and row
@@ -138,7 +162,7 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
     constexpr int A_BYTES = W::A_BYTES, STAGE_BYTES = W::STAGE_BYTES;
     constexpr int KS = W::KS, KH = W::KH, NM = W::NM, XM = W::XM, XK = W::XK, NTILE = W::NTILE;
     constexpr bool EXTRA = W::EXTRA, EPI = W::EPI;
-    extern __shared__ __attribute__((aligned(1024))) unsigned char wsmem[];  // W::LDS_BYTES
+    extern __shared__ __attribute__((aligned(1024))) unsigned char wsmem[];  // W::LAUNCH_LDS_BYTES
 
     const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
     const unsigned g = lid / tiles_n;
@@ -219,6 +243,21 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
             b_next = Wt + p * b_plane;
         }
     };
+
+    // Lines touched ahead (W::TOUCH): the first step of a position touches the next position's A tiles of up to four
+    // steps, wave w rows 16w .. 16w+15, one lane per 128-byte line.
+    unsigned touch_voff = 0;
+    const unsigned touch_lds = smem_base + W::LDS_BYTES + wave * 256u;
+    if constexpr (W::TOUCH) {
+        const unsigned row = 16u * wave + (lane & 15);
+        unsigned grow;
+        if (row < static_cast<unsigned>(W::BM))
+            grow = row < rows_valid ? row : rows_valid - 1;
+        else
+            grow = has_extra ? xrow0 - m0 + (row - W::BM < xrows_valid ? row - W::BM : xrows_valid - 1) : rows_valid - 1;
+        const unsigned line = static_cast<unsigned>(lane >> 4) < static_cast<unsigned>(nkc) ? lane >> 4 : nkc - 1;
+        touch_voff = grow * static_cast<unsigned>(R) * 4u + line * 128u;
+    }
 
     // ---- MFMA operands --------------------------------------------------------------------------------
     // Per group of 16 channels, lane group lg feeds channels 4*lg .. 4*lg+3, one per MFMA: A is one b128 read
@@ -379,9 +418,11 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
 
     // One step of the q-th position walked, on ring slot `stage`.  first: the position's first step (accumulators
     // start from zero where the schedule says so; the vector work and the stores of the schedule ride along).
-    auto step = [&](auto q_tag, auto first_tag, auto stage_tag) __attribute__((always_inline)) {
+    // after_first: the step before was the position's first (its line touch is still outstanding behind its copies).
+    auto step = [&](auto q_tag, auto first_tag, auto stage_tag, auto after_first_tag) __attribute__((always_inline)) {
         constexpr int q = decltype(q_tag)::value;
         constexpr bool first = decltype(first_tag)::value;
+        constexpr int NTOUCH = W::TOUCH && decltype(after_first_tag)::value ? 1 : 0;
         using Other = std::integral_constant<int, (decltype(stage_tag)::value + 1) % NSTAGE>;   // the next step's slot
         constexpr int dst = kWideDst[q];
         constexpr bool fresh = first && kWideFresh[q];
@@ -443,9 +484,9 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
             mfma_slot(F2, i, false);
             if (i == 0) {
                 // The tile of the next step is complete once nothing but what was issued after its copies is
-                // outstanding: the copies of the steps behind it in the ring and the stores (and residual loads)
-                // of this step's first half.  Memory operations complete in issue order.
-                constexpr int mine = (NSTAGE - 2) * LPS + (store_plane >= 0 ? W::PLANE_OPS : 0);
+                // outstanding: the copies of the steps behind it in the ring, the line touch of the step before and
+                // the stores (and residual loads) of this step's first half.  Memory operations complete in issue order.
+                constexpr int mine = (NSTAGE - 2) * LPS + NTOUCH + (store_plane >= 0 ? W::PLANE_OPS : 0);
                 wait_vmcnt<(mine < 63 ? mine : 63)>();
                 __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS reads of this step are done
                 __builtin_amdgcn_s_barrier();
@@ -454,6 +495,8 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
 #pragma unroll
             for (int c = 0; c < LPS; ++c)
                 if (copy_slot(c) == i) copy(stage_tag, c);
+            if constexpr (W::TOUCH && first && i == NM - 1)  // behind the step's last copy
+                async_touch4(a_base + kWidePos[(q + 1) & 15] * a_plane, touch_voff, touch_lds);
 #pragma unroll
             for (int u = 0; u < NU; ++u)
                 if (read_slot(u) == i) read_unit(F1, Other{}, 0, u);
@@ -475,10 +518,12 @@ __global__ __launch_bounds__(W::NT) __attribute__((amdgpu_waves_per_eu(W::OCC, W
 
     // Steps go round the ring slots; a position has a multiple of NSTAGE steps, so it starts on slot 0.
     static_for<16>([&](auto q_tag) {
-        step(q_tag, std::true_type{}, Stage0{});
-        static_for<NSTAGE - 1>([&](auto s_tag) { step(q_tag, std::false_type{}, std::integral_constant<int, decltype(s_tag)::value + 1>{}); });
+        step(q_tag, std::true_type{}, Stage0{}, std::false_type{});
+        static_for<NSTAGE - 1>([&](auto s_tag) {
+            step(q_tag, std::false_type{}, std::integral_constant<int, decltype(s_tag)::value + 1>{}, std::bool_constant<decltype(s_tag)::value == 0>{});
+        });
         for (int kc = NSTAGE; kc < nkc; kc += NSTAGE)
-            static_for<NSTAGE>([&](auto s_tag) { step(q_tag, std::false_type{}, s_tag); });
+            static_for<NSTAGE>([&](auto s_tag) { step(q_tag, std::false_type{}, s_tag, std::false_type{}); });
     });
 
     // The surplus copies must have landed before this workgroup's LDS can be handed on.
