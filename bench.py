@@ -47,7 +47,7 @@ MEASURED_TRAFFIC = {
     ("cfg2", "bf16_stored", "imtrans"): (None, (25128.0 * 2 + 100352.0) * 1024),
     ("cfg4a", "bf16_stored", "conv"): ("stored-split", (23787.0 * 2 + 12544.0) * 1024),
     ("cfg4a", "bf16_stored", "imtrans"): (None, (6312.0 * 2 + 25088.0) * 1024),
-    ("cfg4b", "bf16_stored", "conv"): ("stored-split4", (45085.0 * 2 + 8192.0) * 1024),
+    ("cfg4b", "bf16_stored", "conv"): ("stored-spread", (24747.7 * 2 + 24576.0) * 1024),   # both kernels
     ("cfg4b", "bf16_stored", "imtrans"): (None, (3176.0 * 2 + 16384.0) * 1024),
 }
 
@@ -298,6 +298,8 @@ def main():
     ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16", "bf16_stored"],
                     help="fp32 (the reference's arithmetic); bf16: GEMM operands rounded to bf16 inside the conv "
                          "kernel; bf16_stored: the transformed activations are also written and read as bf16")
+    ap.add_argument("--no-workspace", action="store_true",
+                    help="bf16_stored: call the convolution without its scratch buffer (swc_winograd2x2_conv_bf16in)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg and the parity gate")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU work for cpu_baseline")
     ap.add_argument("--backward", action="store_true",
@@ -381,8 +383,13 @@ def main():
         def call_imtrans(a, b, st):
             return L.swc_winograd2x2_imtrans_bf16out(a, None, None, b, C, B, H, W, 1, 1, 1, st)
 
+        # the launcher's scratch buffer (what tmp_data_buffer is to the reference's launcher), allocated once
+        ws_floats = 0 if args.no_workspace else L.swc_winograd2x2_conv_bf16in_workspace_floats(C, B, nH, nW, K)
+        ws = torch.empty(max(ws_floats, 1), dtype=torch.float32, device=dev)
+        wsp = ws.data_ptr() if ws_floats else None
+
         def call_conv(b, c, st):
-            return L.swc_winograd2x2_conv_bf16in(b, w16p, c, None, None, None, 0, C, B, nH, nW, K, 1, 1, st)
+            return L.swc_winograd2x2_conv_bf16in_ws(b, w16p, c, None, None, None, 0, wsp, ws_floats, C, B, nH, nW, K, 1, 1, st)
     else:
         conv_entry = L.swc_winograd2x2_conv if args.precision == "fp32" else L.swc_winograd2x2_conv_bf16
         winograd2x2_imTrans(x, relu=True, out=ti)

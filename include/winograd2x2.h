@@ -14,6 +14,7 @@
 #ifndef WINOGRAD2X2_H_
 #define WINOGRAD2X2_H_
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -41,7 +42,7 @@ SWC_API int swc_last_hip_error(void);
 /* Library version, "major.minor". */
 SWC_API const char *swc_version(void);
 /* Diagnostic with no counterpart in the reference: the name of the convolution kernel that the calling
- * thread's last swc_winograd2x2_conv / _conv_bf16 / _conv_epilogue / _conv_bf16in call launched ("" before the
+ * thread's last swc_winograd2x2_conv / _conv_bf16 / _conv_epilogue / _conv_bf16in / _conv_bf16in_ws call launched ("" before the
  * first): "sync" (any shape and alignment), "ring32" / "ring16" (64x64 tiles, 32- / 16-channel steps),
  * "tall16" / "short16" (row groups of up to 112 / 32 rows, dealt evenly over the CUs), "wide48" (48 rows x 128
  * columns per workgroup, left-over rows as extra tiles split along the channels; C % 64 == 0, K % 128 == 0),
@@ -49,10 +50,12 @@ SWC_API const char *swc_version(void);
  * bf16-stored operands "stored-ring3" / "stored-ring4" (64x64 tiles, 3- / 4-deep copy ring) / "stored-split"
  * (small grids: the 16 positions of a tile split over two groups of waves, whose partial sums are added at the
  * end) / "stored-split4" (smaller grids still: 32-row tiles, four groups of waves) / "stored-tall" (128x64
- * tiles for C = 64, 128, 256 or 512 on grids that fill the device).  Which one runs depends only on the shapes,
- * pointer alignment and the device's CU count and L2 size; all give the same results to within the order of
- * the fp32 summations ("wide48" and "stored-tall" also add the nine terms of an output in another order than
- * the rest: 1e-6 relative, exact on integer-valued data). */
+ * tiles for C = 64, 128, 256 or 512 on grids that fill the device) / "stored-spread" (the same tiles, four workgroups
+ * each, on grids far too small for it; swc_winograd2x2_conv_bf16in_ws with a scratch buffer only).  Which one runs
+ * depends only on the shapes, pointer alignment, whether a scratch buffer was passed, and the device's CU count and
+ * L2 size; all give the same results to within the order of the fp32 summations ("wide48", "stored-tall" and
+ * "stored-spread" also add the nine terms of an output in another order than the rest: 1e-6 relative, exact on
+ * integer-valued data). */
 SWC_API const char *swc_winograd2x2_conv_last_kernel(void);
 /* Diagnostic with no counterpart in the reference, for benchmarks and tests that compare the tilings: makes
  * the calling thread's later swc_winograd2x2_conv calls
@@ -231,6 +234,22 @@ SWC_API int swc_winograd2x2_weights_bf16(const float *Weight, uint16_t *Weight16
 SWC_API int swc_winograd2x2_conv_bf16in(const uint16_t *Input16, const uint16_t *Weight16t, float *Output,
                                 const float *Scale, const float *Shift, const float *Residual, int residual_relu,
                                 int C, int B, int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream);
+
+/* swc_winograd2x2_conv_bf16in with a scratch buffer of the caller's (device memory, 16-byte aligned): what the
+ * reference's tmp_data_buffer is to its launcher (winograd2x2_conv_op.cc:57-60 allocates 16*M*K floats per call,
+ * winograd2x2_conv_cuda.cu.cc:65 takes them).  Layers of 256 or 512 channels with so few 128-row x 64-column tiles
+ * that four times as many workgroups still find a CU each (7x7x512 at batch 64, 14x14x256 at batch 16) then run as
+ * four workgroups per tile, one per row of the 4x4 position grid,
+ * whose partial sums meet in the buffer; a second kernel combines them, applies the epilogue and writes the output.
+ * swc_winograd2x2_conv_bf16in_workspace_floats says how many floats that takes on the current device (8*M*K, or 0
+ * for shapes that do not use a buffer).  With Workspace NULL, or fewer than that many floats, the call is
+ * swc_winograd2x2_conv_bf16in.  The sums of the output transform are then taken row by row of the position grid:
+ * results agree with swc_winograd2x2_conv_bf16in to rounding, not bit for bit. */
+SWC_API size_t swc_winograd2x2_conv_bf16in_workspace_floats(int C, int B, int nH, int nW, int K);
+SWC_API int swc_winograd2x2_conv_bf16in_ws(const uint16_t *Input16, const uint16_t *Weight16t, float *Output,
+                                   const float *Scale, const float *Shift, const float *Residual, int residual_relu,
+                                   float *Workspace, size_t workspace_floats,
+                                   int C, int B, int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream);
 
 /* The whole layer in one kernel with bf16 GEMM operands: the values of swc_winograd2x2_imtrans_bf16out
  * (with InScale/InShift as in swc_winograd2x2_imtrans_affine, or NULL) followed by

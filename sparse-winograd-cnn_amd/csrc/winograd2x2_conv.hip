@@ -156,12 +156,58 @@ int launch_bf16_stored(const unsigned short *Input16, const unsigned short *Weig
 }  // namespace
 }  // namespace swc
 
+namespace swc {
+namespace {
+// Layers of 256 or 512 channels with so few 128-row x 64-column tiles that four workgroups per tile still find a CU
+// each: with a scratch buffer the positions of a tile are dealt over four workgroups.  With 256 channels a workgroup's
+// four positions are 16 steps only and the second kernel weighs twice as much: the form pays up to half as many
+// workgroups (14x14x256 -> 256 at batch 16: 11.8 us against 14.8; at batch 32, 208 workgroups: 16.5 against 15.2;
+// 7x7x512 -> 512 at batch 64, 256 workgroups: 18.5 against 23.9; at batch 128: 34.1 against 30.8).
+bool bf16_spread_wanted(size_t M, int C, int K, size_t cus)
+{
+    if ((C != 256 && C != 512) || K % 64 != 0) return false;
+    const size_t tall_n = static_cast<size_t>(K) / 64, tall_m = (M + 127) / 128;
+    return 4 * tall_m * tall_n * static_cast<size_t>(512 / C) <= cus;
+}
+int conv_bf16in(const unsigned short *Input16, const unsigned short *Weight16t, float *Output, const float *Scale,
+                const float *Shift, const float *Residual, int residual_relu, float *Workspace, size_t workspace_floats, int C,
+                int B, int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream);
+}  // namespace
+}  // namespace swc
+
 extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const unsigned short *Weight16t, float *Output,
                                            const float *Scale, const float *Shift, const float *Residual,
                                            int residual_relu, int C, int B, int nH, int nW, int K, int pad_h, int pad_w,
                                            swc_stream_t stream)
 {
+    return swc::conv_bf16in(Input16, Weight16t, Output, Scale, Shift, Residual, residual_relu, nullptr, 0, C, B, nH, nW, K, pad_h,
+                            pad_w, stream);
+}
+
+extern "C" size_t swc_winograd2x2_conv_bf16in_workspace_floats(int C, int B, int nH, int nW, int K)
+{
     using namespace swc;
+    if (C <= 0 || B <= 0 || nH <= 0 || nW <= 0 || K <= 0) return 0;
+    const size_t M = static_cast<size_t>(B) * nH * nW;
+    if (M >= (1ull << 31) || M * 16 * static_cast<size_t>(K) >= (1ull << 31)) return 0;
+    return bf16_spread_wanted(M, C, K, device_cus()) ? 8 * M * static_cast<size_t>(K) : 0;
+}
+
+extern "C" int swc_winograd2x2_conv_bf16in_ws(const unsigned short *Input16, const unsigned short *Weight16t, float *Output,
+                                              const float *Scale, const float *Shift, const float *Residual,
+                                              int residual_relu, float *Workspace, size_t workspace_floats, int C, int B,
+                                              int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream)
+{
+    return swc::conv_bf16in(Input16, Weight16t, Output, Scale, Shift, Residual, residual_relu, Workspace, workspace_floats, C, B, nH,
+                            nW, K, pad_h, pad_w, stream);
+}
+
+namespace swc {
+namespace {
+int conv_bf16in(const unsigned short *Input16, const unsigned short *Weight16t, float *Output, const float *Scale,
+                const float *Shift, const float *Residual, int residual_relu, float *Workspace, size_t workspace_floats, int C,
+                int B, int nH, int nW, int K, int pad_h, int pad_w, swc_stream_t stream)
+{
     if (Input16 == nullptr || Weight16t == nullptr || Output == nullptr) return SWC_ERR_NULL_POINTER;
     if ((Scale == nullptr) != (Shift == nullptr)) return SWC_ERR_NULL_POINTER;
     if (C <= 0 || B <= 0 || nH <= 0 || nW <= 0 || K <= 0) return SWC_ERR_BAD_DIMS;
@@ -210,6 +256,13 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
             return launch_bf16_tall(Input16, Weight16t, Output, M, C, K, nW, tall_rows, Scale, Shift, Residual, residual_relu != 0, s);
         }
     }
+    // Far fewer tiles than that, 256 or 512 channels and a scratch buffer of the caller's: four workgroups per tile,
+    // each a row of the position grid (7x7x512 at batch 64: 18.5 us, 23.9 without the buffer).
+    if (Workspace != nullptr && bf16_spread_wanted(M, C, K, cus) && workspace_floats >= 8 * M * static_cast<size_t>(K) &&
+        bf16_spread_eligible(Input16, Weight16t, Output, Workspace, M, C, K, Scale, Shift, Residual)) {
+        note_conv_kernel("stored-spread");
+        return launch_bf16_spread(Input16, Weight16t, Output, Workspace, M, C, K, nW, Scale, Shift, Residual, residual_relu != 0, s);
+    }
     // A grid of full tiles that leaves every CU with one workgroup at most: the launch then lasts as long as one
     // workgroup's chain of steps, and splitting the 16 positions over two groups of waves halves the chain
     // (7x7x512 at batch 64: 30.7 us against 37.1; 14x14x256: 19.9 against 22.9).
@@ -235,3 +288,5 @@ extern "C" int swc_winograd2x2_conv_bf16in(const unsigned short *Input16, const 
     note_conv_kernel("stored-ring4");
     return launch_bf16_stored<Deep>(Input16, Weight16t, Output, M, C, K, nH, nW, rows, tiles_n, ep, s);
 }
+}  // namespace
+}  // namespace swc

@@ -54,10 +54,16 @@ __device__ __forceinline__ void lds_copy_run2(unsigned v0, unsigned v1, const ch
 }
 
 // NKC 64-channel steps per position (C = 64*NKC), OCC waves per SIMD, EPI: scale/shift/residual in the stores.
-template <int NKC_, int OCC_, bool EPI_>
+// SPREAD: the 16 positions of a tile are dealt over four workgroups, one per row r of the 4x4 position grid; each
+// writes the two partial sums Z_r(dx) = sum_s a_dx[s] P[r][s] of its tile as planes [r][dx][M][K] of a scratch buffer,
+// and spread_combine_kernel takes Y(dy,dx) = sum_r a_dy[r] Z_r(dx) from there.  For layers with too few tiles for the
+// CUs: a quarter of the bytes per workgroup through LDS, and every byte of the operands fetched by one XCD only.
+template <int NKC_, int OCC_, bool EPI_, bool SPREAD_ = false>
 struct TallCfg {
     static constexpr int NKC = NKC_, OCC = OCC_, NSTAGE = 3;
-    static constexpr bool EPI = EPI_, EARLY = !EPI_;
+    static constexpr bool EPI = EPI_, EARLY = !EPI_, SPREAD = SPREAD_;
+    static constexpr int NQ = SPREAD ? 4 : 16;           // positions a workgroup walks
+    static_assert(!SPREAD || !EPI, "the epilogue of a spread launch is applied by the combining kernel");
     static constexpr int BM = 128, BN = 64, BK = 64, NT = 256, TM = 2;
     static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
@@ -77,7 +83,8 @@ struct TallCfg {
 };
 
 // Requirements checked by the launcher: C == 64*NKC, K % 64 == 0, TI16 and Wt16 16-byte aligned, M*C*2 < 2^32, the
-// output below 2^31 bytes.  grid.x = ceil(M / rows_per_wg) * (K / 64), rows_per_wg <= 128.
+// output below 2^31 bytes.  grid.x = ceil(M / rows_per_wg) * (K / 64), rows_per_wg <= 128; with SPREAD four times
+// that (workgroup lid takes row lid / (grid.x / 4) of the position grid) and Out is the scratch buffer, 8*M*K floats.
 template <typename T>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::OCC, T::OCC))) void conv_bf16_tall_kernel(
     const unsigned short *__restrict__ TI16, const unsigned short *__restrict__ Wt16, float *__restrict__ Out, unsigned M,
@@ -88,7 +95,10 @@ __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::OCC, T
     constexpr bool EPI = T::EPI;
     extern __shared__ __attribute__((aligned(1024))) unsigned char tsmem[];  // T::LDS_BYTES
 
-    const unsigned lid = xcd_swizzle(blockIdx.x, gridDim.x);
+    const unsigned lid_all = xcd_swizzle(blockIdx.x, gridDim.x);
+    const unsigned tiles_all = T::SPREAD ? gridDim.x / 4 : gridDim.x;
+    const unsigned grid_row = T::SPREAD ? lid_all / tiles_all : 0;  // r: this workgroup's positions are 4r .. 4r+3
+    const unsigned lid = T::SPREAD ? lid_all % tiles_all : lid_all;
     const unsigned m0 = (lid / tiles_n) * rows_per_wg;
     const unsigned n0 = (lid % tiles_n) * T::BN;
     const unsigned rows_valid = M - m0 < rows_per_wg ? M - m0 : rows_per_wg;
@@ -130,12 +140,14 @@ __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::OCC, T
         const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(b >> 32));
         return reinterpret_cast<const char *>((static_cast<size_t>(hi) << 32) | lo);
     };
-    // The copies of global step si (position walked (si / NKC) % 16, chunk si % NKC) into ring slot si % NSTAGE.
+    // The copies of global step si (position walked (si / NKC) % NQ, chunk si % NKC) into ring slot si % NSTAGE.
     // Past the last step the walk starts over: the surplus copies land in ring slots nobody reads any more.
+    // A spread workgroup walks the columns of its grid row in the order of the walk's first row (1, 2, 0, 3).
     auto set_issue_position = [&](auto si_tag) __attribute__((always_inline)) {
         constexpr int si = decltype(si_tag)::value;
         if constexpr (si % NKC == 0) {
-            constexpr size_t pos = kWidePos[(si / NKC) % 16];
+            constexpr size_t walked = kWidePos[(si / NKC) % T::NQ];
+            const size_t pos = T::SPREAD ? 4 * grid_row + (walked & 3) : walked;
             a_ptr = scalar_ptr(a_base + pos * a_plane);
             b_ptr = scalar_ptr(b_base + pos * b_plane);
         }
@@ -177,14 +189,20 @@ __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::OCC, T
     const unsigned oW = 2u * static_cast<unsigned>(nW);
     const unsigned row_stride = oW * static_cast<unsigned>(K);  // floats
     const unsigned out_bytes = M * 4u * static_cast<unsigned>(K) * 4u;
-    const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(Out, out_bytes);
+    // spread: the two planes [grid_row][0..1][M][K] of the scratch buffer, rows addressed by tile row
+    const unsigned part_plane_bytes = M * static_cast<unsigned>(K) * 4u;
+    const __amdgpu_buffer_rsrc_t out_rsrc = T::SPREAD ? make_rsrc(Out + static_cast<size_t>(2 * grid_row) * M * K, 2 * part_plane_bytes)
+                                                      : make_rsrc(Out, out_bytes);
     const __amdgpu_buffer_rsrc_t res_rsrc = make_rsrc(ep.residual, EPI && ep.residual != nullptr ? out_bytes : 0u);
     unsigned *const rowoff = reinterpret_cast<unsigned *>(tsmem);
     if (tid < T::BM) {
         const unsigned gm = m0 + tid;
         const unsigned bt = gm / static_cast<unsigned>(nW);
         const unsigned tw = gm - bt * static_cast<unsigned>(nW);
-        rowoff[tid] = static_cast<unsigned>(tid) < rows_valid ? (bt * 2u * oW + 2u * tw) * static_cast<unsigned>(K) * 4u : kWideOutOfRange;
+        if constexpr (T::SPREAD)
+            rowoff[tid] = static_cast<unsigned>(tid) < rows_valid ? gm * static_cast<unsigned>(K) * 4u : kWideOutOfRange;
+        else
+            rowoff[tid] = static_cast<unsigned>(tid) < rows_valid ? (bt * 2u * oW + 2u * tw) * static_cast<unsigned>(K) * 4u : kWideOutOfRange;
     }
     const unsigned col = n0 + 32 * wn + li;
     const unsigned col_bytes = col * 4u;
@@ -342,10 +360,30 @@ __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::OCC, T
         });
     };
 
-    static_for<16>([&](auto q_tag) { static_for<NKC>([&](auto kc_tag) { step(q_tag, kc_tag); }); });
+    static_for<T::NQ>([&](auto q_tag) { static_for<NKC>([&](auto kc_tag) { step(q_tag, kc_tag); }); });
 
     // The surplus copies must have landed before this workgroup's LDS can be handed on.
     wait_vmcnt<0>();
+
+    if constexpr (T::SPREAD) {
+        // After the four positions of a grid row set 2 holds P[r][0] + P[r][1] + P[r][2] = Z_r(0) and set 1
+        // P[r][2] + P[r][3] - P[r][1] = -Z_r(1) (kWideOps, q = 0 .. 3).
+#pragma unroll
+        for (int dx = 0; dx < 2; ++dx)
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const uint4 ro = quarter_offsets(tm, v);
+                    const unsigned off[4] = {ro.x, ro.y, ro.z, ro.w};
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float val = dx == 0 ? S[2][tm][4 * v + r] : -S[1][tm][4 * v + r];
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), out_rsrc, off[r] + col_bytes, dx * part_plane_bytes, 16);
+                    }
+                }
+        return;
+    }
 
     // What has not been stored yet: plane 3, or all four.  With a residual, the values of a plane are read in one
     // sweep before its stores and one plane ahead (loads and stores complete in issue order).

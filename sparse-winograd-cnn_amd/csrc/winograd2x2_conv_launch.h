@@ -108,6 +108,11 @@ inline WidePlan plan_wide48(size_t M, int N, size_t cus, int bn = 128)
 
 // Defined in winograd2x2_conv_bf16_tall.hip: the bf16-stored convolution over 128-row x 64-column tiles.
 bool bf16_tall_eligible(const void *TI16, const void *Wt16, size_t M, int C, int K);
+// The spread form of the same kernel (winograd2x2_conv_bf16_spread.hip): Part is a scratch buffer of 8*M*K floats.
+bool bf16_spread_eligible(const void *TI16, const void *Wt16, const void *Out, const void *Part, size_t M, int C, int K,
+                          const float *scale, const float *shift, const float *residual);
+int launch_bf16_spread(const unsigned short *TI16, const unsigned short *Wt16, float *Out, float *Part, size_t M, int C, int K,
+                       int nW, const float *scale, const float *shift, const float *residual, int residual_relu, hipStream_t stream);
 int launch_bf16_tall(const unsigned short *TI16, const unsigned short *Wt16, float *Out, size_t M, int C, int K, int nW,
                      size_t rows_per_wg, const float *scale, const float *shift, const float *residual, int residual_relu,
                      hipStream_t stream);

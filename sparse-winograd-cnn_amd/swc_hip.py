@@ -26,6 +26,7 @@ C_SYMBOLS = (
     "swc_winograd2x2_imtrans", "swc_winograd2x2_imtrans_affine", "swc_winograd2x2_conv", "swc_winograd2x2_conv_bf16",
     "swc_winograd2x2_conv_epilogue",
     "swc_winograd2x2_imtrans_bf16out", "swc_winograd2x2_weights_bf16", "swc_winograd2x2_conv_bf16in",
+    "swc_winograd2x2_conv_bf16in_ws", "swc_winograd2x2_conv_bf16in_workspace_floats",
     "swc_winograd2x2_relu_conv_bf16",
     "swc_winograd2x2_imtrans_op_shape", "swc_winograd2x2_imtrans_op_compute",
     "swc_winograd2x2_conv_op_shape", "swc_winograd2x2_conv_op_compute",
@@ -99,6 +100,10 @@ def lib():
         L.swc_winograd2x2_weights_bf16.argtypes = [fp, fp, i32, i32, vp]
         L.swc_winograd2x2_conv_bf16in.restype = i32
         L.swc_winograd2x2_conv_bf16in.argtypes = [fp] * 6 + [i32] * 8 + [vp]
+        L.swc_winograd2x2_conv_bf16in_ws.restype = i32
+        L.swc_winograd2x2_conv_bf16in_ws.argtypes = [fp] * 6 + [i32, fp, ctypes.c_size_t] + [i32] * 7 + [vp]
+        L.swc_winograd2x2_conv_bf16in_workspace_floats.restype = ctypes.c_size_t
+        L.swc_winograd2x2_conv_bf16in_workspace_floats.argtypes = [i32] * 5
         L.swc_winograd2x2_relu_conv_bf16.restype = i32
         L.swc_winograd2x2_relu_conv_bf16.argtypes = [fp] * 8 + [i32] * 8 + [vp]
         L.swc_winograd2x2_imtrans_op_shape.restype = i32

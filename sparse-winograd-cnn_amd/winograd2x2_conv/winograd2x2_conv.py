@@ -96,7 +96,7 @@ def winograd2x2_weights_bf16(W):
     return out
 
 
-def _forward_bf16_stored(I, W, out, scale, shift, residual, residual_relu=False):
+def _forward_bf16_stored(I, W, out, scale, shift, residual, residual_relu=False, workspace=True):
     """I [16,B,nH,nW,C] bfloat16; W [16,C,K] float32 or prepared [16,K,C] bfloat16."""
     I = swc_hip.require_cuda_f32(I, "I", 5, torch.bfloat16)
     if not isinstance(W, torch.Tensor) or W.dim() != 3:
@@ -125,10 +125,15 @@ def _forward_bf16_stored(I, W, out, scale, shift, residual, residual_relu=False)
         if tuple(residual.shape) != shape:
             raise ValueError("residual must have the output's shape %s" % (shape,))
     with swc_hip.on_device(I.device) as stream:
-        st = swc_hip.lib().swc_winograd2x2_conv_bf16in(
+        L = swc_hip.lib()
+        # the launcher's temporary, allocated per call as the reference's op does (winograd2x2_conv_op.cc:57-60);
+        # most shapes need none
+        tmp_floats = L.swc_winograd2x2_conv_bf16in_workspace_floats(C, B, nH, nW, K) if workspace else 0
+        tmp = torch.empty(tmp_floats, dtype=torch.float32, device=I.device) if tmp_floats else None
+        st = L.swc_winograd2x2_conv_bf16in_ws(
             I.data_ptr(), W.data_ptr(), out.data_ptr(), None if scale is None else scale.data_ptr(),
             None if shift is None else shift.data_ptr(), None if residual is None else residual.data_ptr(),
-            int(bool(residual_relu)), C, B, nH, nW, K, 1, 1, stream)
+            int(bool(residual_relu)), None if tmp is None else tmp.data_ptr(), tmp_floats, C, B, nH, nW, K, 1, 1, stream)
     swc_hip.check(st, "winograd2x2_conv (bf16-stored operands)")
     return out
 
@@ -177,7 +182,8 @@ class _ConvFunction(torch.autograd.Function):
         return dI, dW, None
 
 
-def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, residual=None, residual_relu=False):
+def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, residual=None, residual_relu=False,
+                     workspace=True):
     """I: [16,B,nH,nW,C], W: [16,C,K], float32 on the GPU -> [B,2nH,2nW,K] (uncropped).
 
     A bfloat16 ``I`` (from ``winograd2x2_imTrans(..., out_dtype=torch.bfloat16)``) takes the bf16-stored
@@ -188,6 +194,9 @@ def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, r
     residual add that follow the second convolution of a ResNet unit); with ``residual_relu=True`` it is
     ``... + relu(residual)`` (the identity shortcut of the reference model is ``relu(x)``).
 
+    The bf16-stored kernel gets a temporary of the size its launcher asks for (most shapes: none), as the
+    reference's op allocates its launcher's (winograd2x2_conv_op.cc:57-60); ``workspace=False`` calls it without.
+
     ``precision="bf16"`` rounds both GEMM operands to bf16 (fp32 accumulate).  Differentiable
     through ``winograd2x2_conv_grad`` when an input requires grad.
     """
@@ -195,7 +204,7 @@ def winograd2x2_conv(I, W, precision="fp32", out=None, scale=None, shift=None, r
     if isinstance(I, torch.Tensor) and I.dtype == torch.bfloat16:
         if needs_grad:
             raise NotImplementedError("the bf16-stored variant is forward only")
-        return _forward_bf16_stored(I, W, out, scale, shift, residual, residual_relu)
+        return _forward_bf16_stored(I, W, out, scale, shift, residual, residual_relu, workspace)
     if residual_relu and residual is None:
         raise ValueError("residual_relu needs a residual")
     if (scale is not None or residual is not None) and needs_grad:

@@ -81,12 +81,15 @@ def rel_l1(a, b):
     return float(np.sum(np.abs(a - b)) / (den if den > 0 else 1.0))
 
 
-def expected_stored_launch(M, C, K, cus, l2_bytes):
-    """The launch form swc_winograd2x2_conv_bf16in picks for tile rows M, channels C, filters K on a device with
-    `cus` compute units and L2s of `l2_bytes` (the rules of its launcher, restated), as a one-element tuple."""
+def expected_stored_launch(M, C, K, cus, l2_bytes, workspace=True):
+    """The launch form swc_winograd2x2_conv_bf16in_ws (swc_winograd2x2_conv_bf16in with workspace=False) picks for
+    tile rows M, channels C, filters K on a device with `cus` compute units and L2s of `l2_bytes` (the rules of
+    its launcher, restated), as a one-element tuple."""
     ceil = lambda a, b: -(-a // b)
     if C in (64, 128, 256, 512) and K % 64 == 0 and ceil(M, 128) * (K // 64) * 4 >= 3 * cus:
         return ("stored-tall",)
+    if workspace and C in (256, 512) and K % 64 == 0 and 4 * ceil(M, 128) * (K // 64) * (512 // C) <= cus:
+        return ("stored-spread",)
     if ceil(M, 32) * ceil(K, 64) <= cus and C >= 256:
         return ("stored-split4",)
     if ceil(M, 64) * ceil(K, 64) <= cus:

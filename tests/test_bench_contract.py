@@ -53,7 +53,7 @@ def _profile_traffic_tables():
     import re
 
     variants = {"wide48x64": "wide48x64", "wide48": "wide48", "tall16": "tall16", "short16": "short16", "ring32": "ring32", "ring16": "ring16",
-                "3-ring": "stored-ring3", "4-ring": "stored-ring4", "stored-split4": "stored-split4",
+                "3-ring": "stored-ring3", "4-ring": "stored-ring4", "stored-spread": "stored-spread", "stored-split4": "stored-split4",
                 "stored-split`": "stored-split", "stored-tall": "stored-tall"}
     out = {}
     for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "conv_imtrans_*.md"))):

@@ -115,14 +115,63 @@ def test_stored_split4_kernel(oracle, dev, shape):
     w = (rng.standard_normal((16, C, K)) * 0.05).astype(np.float32)
     ti16, w16 = oracle.round_bf16(ti), oracle.round_bf16(w)
     ti_gpu, w_gpu = gpu(ti16, dev).to(torch.bfloat16), winograd2x2_weights_bf16(gpu(w, dev))
-    got = winograd2x2_conv(ti_gpu, w_gpu).cpu().numpy()
+    got = winograd2x2_conv(ti_gpu, w_gpu, workspace=False).cpu().numpy()
     assert swc_hip.lib().swc_winograd2x2_conv_last_kernel() == b"stored-split4"
     want = oracle.conv(ti16, w16, acc64=True)
     assert got.shape == want.shape
     assert rel_max(got, want) <= TOL
     ti_i = rng.integers(-3, 4, size=ti.shape).astype(np.float32)
     w_i = rng.integers(-3, 4, size=w.shape).astype(np.float32)
+    got_i = winograd2x2_conv(gpu(ti_i, dev).to(torch.bfloat16), gpu(w_i, dev), workspace=False).cpu().numpy()
+    assert np.array_equal(got_i, oracle.conv(ti_i, w_i))
+    scale = (0.5 + rng.random(K)).astype(np.float32) * rng.choice([-1, 1], K).astype(np.float32)
+    shift = rng.standard_normal(K).astype(np.float32)
+    res = rng.standard_normal(want.shape).astype(np.float32)
+    got2 = winograd2x2_conv(ti_gpu, w_gpu, scale=gpu(scale, dev), shift=gpu(shift, dev), residual=gpu(res, dev),
+                            workspace=False).cpu().numpy()
+    assert np.array_equal(got2, oracle.affine(got, scale, shift) + res)
+    got3 = winograd2x2_conv(ti_gpu, w_gpu, residual=gpu(res, dev), residual_relu=True, workspace=False).cpu().numpy()
+    assert np.array_equal(got3, got + np.maximum(res, 0))
+
+
+@pytest.mark.parametrize("shape", [
+    (64, 4, 4, 512, 512),    # config 4b: 8 x 8 tiles of 128 rows x 64 columns, four workgroups each
+    (16, 7, 7, 256, 256),    # M = 784: the last row group holds 16 rows; four steps per position
+    (3, 5, 7, 256, 128),     # M = 105: one ragged row group
+    (1, 1, 1, 512, 64),      # one row
+    (5, 9, 9, 512, 192),     # M = 405
+])
+def test_stored_spread_kernel(oracle, dev, shape):
+    """Layers of 256 or 512 channels with too few 128-row x 64-column tiles for the chip, given a scratch buffer, run
+    `stored-spread` (four workgroups per tile, one per row of the position grid; a second kernel combines their
+    partial sums): values against the oracle fed the same bf16 operands, exactly on integers (every sign, the
+    scatter), the epilogue's arithmetic exactly, and the entry point's fallback without a buffer."""
+    import swc_hip
+    from winograd2x2_conv.winograd2x2_conv import winograd2x2_conv, winograd2x2_weights_bf16
+    B, nH, nW, C, K = shape
+    L = swc_hip.lib()
+    M = B * nH * nW
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    if 4 * -(-M // 128) * (K // 64) * (512 // C) > cus:
+        pytest.skip("this device has too few CUs for the shape to take the spread form")
+    assert L.swc_winograd2x2_conv_bf16in_workspace_floats(C, B, nH, nW, K) == 8 * M * K
+    rng = np.random.default_rng(69)
+    ti = np.maximum(rng.standard_normal((16, B, nH, nW, C)), 0).astype(np.float32)
+    w = (rng.standard_normal((16, C, K)) * 0.05).astype(np.float32)
+    ti16, w16 = oracle.round_bf16(ti), oracle.round_bf16(w)
+    ti_gpu, w_gpu = gpu(ti16, dev).to(torch.bfloat16), winograd2x2_weights_bf16(gpu(w, dev))
+    got = winograd2x2_conv(ti_gpu, w_gpu).cpu().numpy()
+    assert L.swc_winograd2x2_conv_last_kernel() == b"stored-spread"
+    want = oracle.conv(ti16, w16, acc64=True)
+    assert got.shape == want.shape
+    assert rel_max(got, want) <= TOL
+    plain = winograd2x2_conv(ti_gpu, w_gpu, workspace=False).cpu().numpy()
+    assert L.swc_winograd2x2_conv_last_kernel() != b"stored-spread"
+    assert rel_max(got, plain) <= 1e-5
+    ti_i = rng.integers(-3, 4, size=ti.shape).astype(np.float32)
+    w_i = rng.integers(-3, 4, size=w.shape).astype(np.float32)
     got_i = winograd2x2_conv(gpu(ti_i, dev).to(torch.bfloat16), gpu(w_i, dev)).cpu().numpy()
+    assert L.swc_winograd2x2_conv_last_kernel() == b"stored-spread"
     assert np.array_equal(got_i, oracle.conv(ti_i, w_i))
     scale = (0.5 + rng.random(K)).astype(np.float32) * rng.choice([-1, 1], K).astype(np.float32)
     shift = rng.standard_normal(K).astype(np.float32)
@@ -131,6 +180,14 @@ def test_stored_split4_kernel(oracle, dev, shape):
     assert np.array_equal(got2, oracle.affine(got, scale, shift) + res)
     got3 = winograd2x2_conv(ti_gpu, w_gpu, residual=gpu(res, dev), residual_relu=True).cpu().numpy()
     assert np.array_equal(got3, got + np.maximum(res, 0))
+    # a buffer that is too small is not used
+    y = torch.empty(B, 2 * nH, 2 * nW, K, device=dev)
+    small = torch.empty(8 * M * K - 1, device=dev)
+    st = L.swc_winograd2x2_conv_bf16in_ws(ti_gpu.data_ptr(), w_gpu.data_ptr(), y.data_ptr(), None, None, None, 0,
+                                          small.data_ptr(), small.numel(), C, B, nH, nW, K, 1, 1,
+                                          torch.cuda.current_stream().cuda_stream)
+    assert st == 0 and L.swc_winograd2x2_conv_last_kernel() != b"stored-spread"
+    assert np.array_equal(y.cpu().numpy(), plain)
 
 
 @pytest.mark.parametrize("shape", [
